@@ -1,6 +1,7 @@
 // Attention whose scores carry more terms than the product of query and key, and
 // whose values may be narrower or wider than its keys.  For the query of head h at
-// position p and the key at position j <= p (and j > p - W with a window W):
+// position p and the key at position j <= p (and, with a window W, j > p - W or j < F, the
+// first F positions staying visible beside the window):
 //
 //   s(p, j) = (q . k) * scale - slope[h] * (p - j)           (slope: optional, one a head)
 //   w(p, j) = exp(s(p, j)) / (exp(sink[h]) + sum_j' exp(s(p, j')))
@@ -26,6 +27,7 @@ constexpr int SC_MAX_D = 256;
 struct ScoreTerms {
   float scale;
   int window;              // 0: none
+  int keep_first;          // with a window: positions 0 .. keep_first - 1 stay visible beside it
   const float* slopes;     // [nq] or null
   const float* sinks;      // [nq] or null
   const float* gate;       // [n, nq] or null
@@ -68,12 +70,17 @@ attn_scored_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_new, c
 #pragma unroll
   for (int i = 0; i < SC_MAX_D / WAVE; ++i) acc[i] = 0.f;
 
-  for (int j0 = lo; j0 <= p; j0 += WAVE) {
+  // the keys that are seen: the first ones that stay visible beside the window, then the window
+  const int kept = terms.keep_first < lo ? terms.keep_first : lo;
+  for (int part = 0; part < 2; ++part) {
+  const int begin = part == 0 ? 0 : lo;
+  const int end = part == 0 ? kept : p + 1;
+  for (int j0 = begin; j0 < end; j0 += WAVE) {
     const int j = j0 + lane;
     float s = -INFINITY;
     const T* vp = nullptr;
     int vstride = 1;                 // values: [dv][PAGE] in a page, [dv] in the step's rows
-    if (j <= p) {
+    if (j < end) {
       const T* kp;
       if (j < cached) {
         const int page = table[(size_t)b * table_stride + (j / PAGE) % ring_pages];
@@ -91,7 +98,7 @@ attn_scored_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_new, c
       s = dot * terms.scale - slope * (float)(p - j);
     }
     const float m_new = fmaxf(m, wave_max(s));       // finite: key j0 is visible
-    const float pj = (j <= p) ? expf(s - m_new) : 0.f;
+    const float pj = (j < end) ? expf(s - m_new) : 0.f;
     const float alpha = expf(m - m_new);              // 0 in the first tile without a sink (m = -inf)
     l = l * alpha + wave_sum(pj);
     m = m_new;
@@ -100,7 +107,7 @@ attn_scored_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_new, c
     v_s[lane] = vp;
     vstride_s[lane] = vstride;
     __syncthreads();
-    const int cnt = (p - j0 + 1 < WAVE) ? p - j0 + 1 : WAVE;
+    const int cnt = (end - j0 < WAVE) ? end - j0 : WAVE;
 #pragma unroll
     for (int i = 0; i < SC_MAX_D / WAVE; ++i) {
       const int dim = lane + WAVE * i;
@@ -110,6 +117,7 @@ attn_scored_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_new, c
         acc[i] = a;
       }
     }
+  }
   }
   const float g = terms.gate ? terms.gate[(size_t)n * nq + h] : 1.f;
   TO* o = out + ((size_t)n * nq + h) * dv;
@@ -340,19 +348,21 @@ extern "C" {
 int tl_attn_scored_plain(const void* q, const void* k_new, const void* v_new, const void* pages, int dt,
                          const int* table, int table_stride, int ring_pages, const int* row_seq,
                          const int* row_pos, const int* cu_seqlens, const int* n_cached, int n, int nq,
-                         int nkv, int dk, int dv, int window, float scale, const float* slopes,
+                         int nkv, int dk, int dv, int window, int keep_first, float scale, const float* slopes,
                          const float* sinks, const float* gate, void* out, int out_dt, hipStream_t st) {
   TL_REQUIRE(out_dt == dt || out_dt == DT_F32, "scored attention: the result is of the operands' type or float");
   TL_REQUIRE(n >= 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "scored attention: bad head counts nq=%d nkv=%d",
              nq, nkv);
   TL_REQUIRE(dk > 0 && dk <= SC_MAX_D && dv > 0 && dv <= SC_MAX_D,
              "scored attention: head sizes %d and %d are not served (1..%d)", dk, dv, SC_MAX_D);
-  TL_REQUIRE(ring_pages > 0 && table_stride > 0 && window >= 0,
-             "scored attention: bad cache geometry ring_pages=%d table_stride=%d window=%d", ring_pages,
-             table_stride, window);
+  TL_REQUIRE(ring_pages > 0 && table_stride > 0 && window >= 0 && keep_first >= 0,
+             "scored attention: bad cache geometry ring_pages=%d table_stride=%d window=%d keep_first=%d", ring_pages,
+             table_stride, window, keep_first);
+  TL_REQUIRE(keep_first == 0 || window == 0 || (long long)ring_pages * PAGE >= (1LL << 24),
+             "scored attention: first positions that stay visible beside a window need a cache that keeps every position");
   TL_REQUIRE((long long)n * nq < 2147483647LL, "scored attention: too many (row, head) pairs");
   if (n == 0) return 0;
-  const ScoreTerms terms{scale, window, slopes, sinks, gate};
+  const ScoreTerms terms{scale, window, window > 0 ? keep_first : 0, slopes, sinks, gate};
   if (dt == DT_F32)
     attn_scored_plain_kernel<float, float><<<n * nq, 64, 0, st>>>(
         (const float*)q, (const float*)k_new, (const float*)v_new, (const float*)pages, table, table_stride,

@@ -431,7 +431,9 @@ __global__ void rope_commit_kernel(const float* __restrict__ qkv, int n_parts, s
 constexpr int ACT_SILU = 0;
 constexpr int ACT_GELU_TANH = 1;
 constexpr int ACT_SWISH_CLAMPED = 2;   // g' = min(g, limit), u' = clamp(u, -limit, limit): g' logistic(alpha g') (u' + shift)
+constexpr int ACT_RELU = 3;            // max(g, 0)
 __device__ __forceinline__ float gate_act(float g, int act) {
+  if (act == ACT_RELU) return fmaxf(g, 0.f);
   if (act == ACT_GELU_TANH) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
   return g / (1.0f + expf(-g));
 }
@@ -1027,7 +1029,7 @@ int tl_cast_rows(const float* x, long long total, void* out, hipStream_t st) {
 int tl_act_mul(const float* gu, int n, int I, int act, float alpha, float limit, float shift, void* out, int out_dt,
                hipStream_t st) {
   TL_REQUIRE(n >= 0 && I > 0, "act_mul: bad sizes n=%d I=%d", n, I);
-  TL_REQUIRE(act == ACT_SILU || act == ACT_GELU_TANH || act == ACT_SWISH_CLAMPED, "act_mul: no function of code %d", act);
+  TL_REQUIRE(act == ACT_SILU || act == ACT_GELU_TANH || act == ACT_SWISH_CLAMPED || act == ACT_RELU, "act_mul: no function of code %d", act);
   TL_REQUIRE(act != ACT_SWISH_CLAMPED || limit > 0.f, "act_mul: the clamp needs a positive limit");
   if (n == 0) return 0;
   const ActConstants k{alpha, limit, shift};
@@ -1045,7 +1047,7 @@ int tl_act_mul(const float* gu, int n, int I, int act, float alpha, float limit,
 int tl_act_mul_pairs(const void* gu, int n, int I, int act, float alpha, float limit, float shift, void* out,
                      hipStream_t st) {
   TL_REQUIRE(n >= 0 && I > 0 && I % 32 == 0, "act_mul_pairs: bad sizes n=%d I=%d (I in steps of 32)", n, I);
-  TL_REQUIRE(act == ACT_SILU || act == ACT_GELU_TANH || act == ACT_SWISH_CLAMPED, "act_mul_pairs: no function of code %d", act);
+  TL_REQUIRE(act == ACT_SILU || act == ACT_GELU_TANH || act == ACT_SWISH_CLAMPED || act == ACT_RELU, "act_mul_pairs: no function of code %d", act);
   TL_REQUIRE((uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0, "act_mul_pairs: buffers must be 16-byte aligned");
   if (n == 0) return 0;
   const long long chunks = (long long)n * (I / 8);

@@ -52,8 +52,10 @@ constexpr int EPI_GELU_PAIR = 3;    // the same pairs with the tanh form of gelu
                                     // 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))
 constexpr int EPI_SWISH_CLAMPED_PAIR = 4;   // the same pairs with g' = min(g, limit), u' = clamp(u, -limit, limit):
                                             // g' / (1 + exp(-alpha g')) * (u' + shift)
+constexpr int EPI_RELU_PAIR = 5;    // the same pairs with max(g, 0) on the gate
 __host__ __device__ __forceinline__ bool is_pair(int epilogue) {
-  return epilogue == EPI_SILU_PAIR || epilogue == EPI_GELU_PAIR || epilogue == EPI_SWISH_CLAMPED_PAIR;
+  return epilogue == EPI_SILU_PAIR || epilogue == EPI_GELU_PAIR || epilogue == EPI_SWISH_CLAMPED_PAIR ||
+         epilogue == EPI_RELU_PAIR;
 }
 // What happens to the product as the kernels take it: the code, and the constants of a paired epilogue
 // whose function has some.  It reads as its code wherever a plain number is asked for.
@@ -70,6 +72,7 @@ __device__ __forceinline__ float pair_value(float g, float u, const Epi& e) {
     u = fminf(fmaxf(u, -e.limit), e.limit);
     return (g / (1.0f + expf(-e.alpha * g))) * (u + e.shift);
   }
+  if (e.code == EPI_RELU_PAIR) return fmaxf(g, 0.f) * u;
   if (e.code == EPI_GELU_PAIR) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
   return (g / (1.0f + expf(-g))) * u;
 }
@@ -999,7 +1002,7 @@ extern "C" int tl_gemm_bf16(const void* A, const void* W, const void* Wt, int wt
   TL_REQUIRE(K % 8 == 0, "gemm_bf16: K=%d must be a multiple of 8", K);
   TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0) && ((uintptr_t)Wt % 16 == 0),
              "gemm_bf16: operands must be 16-byte aligned");
-  TL_REQUIRE(epilogue >= 0 && epilogue <= 4, "gemm_bf16: unknown epilogue %d", epilogue);
+  TL_REQUIRE(epilogue >= 0 && epilogue <= 5, "gemm_bf16: unknown epilogue %d", epilogue);
   TL_REQUIRE(!is_pair(epilogue) || N % 64 == 0, "gemm_bf16: the paired epilogue needs N=%d to be "
              "a multiple of 64", N);
   if (M == 0) return 0;
@@ -1078,7 +1081,7 @@ extern "C" int tl_gemm_mid_bf16(const void* A, const void* W, void* C, int M, in
   TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_mid: operands must be 16-byte aligned");
   TL_REQUIRE(n_split >= 1 && n_split <= (K + MID_KS - 1) / MID_KS && n_split <= 65535,
              "gemm_mid: %d splits do not fit K=%d (one step of %d at least each)", n_split, K, MID_KS);
-  TL_REQUIRE(epilogue >= 0 && epilogue <= 4 && (n_split == 1 || epilogue == EPI_STORE),
+  TL_REQUIRE(epilogue >= 0 && epilogue <= 5 && (n_split == 1 || epilogue == EPI_STORE),
              "gemm_mid: epilogue %d cannot go with %d splits", epilogue, n_split);
   TL_REQUIRE(!is_pair(epilogue) || N % 64 == 0, "gemm_mid: the paired epilogue needs N=%d to be a "
              "multiple of 64", N);
@@ -1106,7 +1109,7 @@ extern "C" int tl_gemm_ring_bf16(const void* A, const void* W, void* C, int M, i
   TL_REQUIRE(kc == 64 || kc == 128, "gemm_ring: a stage of %d k (64 or 128)", kc);
   TL_REQUIRE(n_split >= 1 && n_split <= K / kc && n_split <= 65535,
              "gemm_ring: %d splits do not fit K=%d (one stage of %d at least each)", n_split, K, kc);
-  TL_REQUIRE(epilogue >= 0 && epilogue <= 4 && (n_split == 1 || epilogue == EPI_STORE),
+  TL_REQUIRE(epilogue >= 0 && epilogue <= 5 && (n_split == 1 || epilogue == EPI_STORE),
              "gemm_ring: epilogue %d cannot go with %d splits", epilogue, n_split);
   TL_REQUIRE(!is_pair(epilogue) || (N % 64 == 0 && waves % 4 == 0), "gemm_ring: the paired epilogue needs N=%d "
              "to be a multiple of 64 and whole groups of four waves (%d)", N, waves);
@@ -1194,7 +1197,7 @@ extern "C" int tl_gemm_bf16_norm(const void* A, const void* W, const void* Wt, i
   TL_REQUIRE(M >= 0 && M <= 16 && N > 0 && K > 0 && K % 8 == 0, "gemm_bf16_norm: bad sizes M=%d N=%d K=%d (at most "
              "16 rows, K a multiple of 8)", M, N, K);
   TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_bf16_norm: operands must be 16-byte aligned");
-  TL_REQUIRE(epilogue >= 0 && epilogue <= 4, "gemm_bf16_norm: unknown epilogue %d", epilogue);
+  TL_REQUIRE(epilogue >= 0 && epilogue <= 5, "gemm_bf16_norm: unknown epilogue %d", epilogue);
   TL_REQUIRE(!is_pair(epilogue) || N % 64 == 0, "gemm_bf16_norm: the paired epilogue needs N=%d to be "
              "a multiple of 64", N);
   TL_REQUIRE(ssq_in == nullptr || n_part > 0, "gemm_bf16_norm: %d partial sums of squares", n_part);

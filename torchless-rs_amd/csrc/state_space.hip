@@ -1,0 +1,270 @@
+// A state-space mixer: a linear recurrence per head over a matrix state, with a short
+// causal convolution before it and a gated, grouped norm behind it.
+//
+// A row of the input projection is [z (inner) | u (C = inner + 2*G*N) | dt (heads)] in float,
+// inner = heads * dv.  u passes a convolution per channel over its last `taps` rows (zeros before
+// the start of a sequence) and silu, and is then read as [x (heads*dv) | B (G*N) | C (G*N)].  With
+// dt' = softplus(dt + dt_bias[h]) and a = exp(-exp(A_log[h]) * dt'), head h (which reads B and C
+// of group h / (heads / G)) keeps a state S [N, dv]:
+//
+//   S <- a S + dt' B x^T ;   y = S^T C + D[h] x
+//
+// and the row's result is rms_parts(y * silu(z)) * w: the gated y cut into equal parts, each
+// divided by its own root mean square (eps inside the root).  dt', a, the state and the sums
+// are float whatever the storage type is; the state lives in a block per sequence,
+// [conv: (taps-1) rows of C channels, the oldest first | S: heads * N * dv], and is carried
+// from step to step.
+#include "common.hpp"
+
+namespace tl {
+
+constexpr int SSM_MAX_TAPS = 8;
+constexpr int SSM_MAX_N = 256;
+constexpr int SSM_MAX_DV = 256;
+constexpr int SSM_TB = 8;              // rows of a sequence that the recurrence stages at a time
+
+__device__ __forceinline__ float silu_f(float a) { return a / (1.0f + expf(-a)); }
+__device__ __forceinline__ float softplus_f(float a) { return fmaxf(a, 0.f) + log1pf(expf(-fabsf(a))); }
+
+// out[n, c] = silu(bias[c] + sum_j w[c, j] * u[row - (taps-1-j), c]); rows before the step come
+// from the sequence's block, rows before the sequence are zeros (the block is zero then).
+template <typename T>
+__global__ void __launch_bounds__(256)
+ssm_conv_kernel(const float* __restrict__ proj, int width, int off, int C, const float* __restrict__ w,
+                const float* __restrict__ bias, int taps, const float* __restrict__ conv_state, long long stride,
+                const int* __restrict__ row_seq, const int* __restrict__ cu_seqlens, const int* __restrict__ slots,
+                T* __restrict__ out) {
+  const int n = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int b = row_seq[n];
+  const int i = n - cu_seqlens[b];
+  const float* old = conv_state + (long long)slots[b] * stride;
+  float acc = bias ? bias[c] : 0.f;
+  for (int j = 0; j < taps; ++j) {
+    const int back = taps - 1 - j;
+    const int src = i - back;
+    const float u = src >= 0 ? proj[(size_t)(n - back) * width + off + c] : old[(size_t)(taps - 1 + src) * C + c];
+    acc = fmaf(w[(size_t)c * taps + j], u, acc);
+  }
+  out[(size_t)n * C + c] = from_f32<T>(silu_f(acc));
+}
+
+// The block's last taps-1 inputs after the step: from the step's rows, or shifted within the block.
+__global__ void __launch_bounds__(256)
+ssm_conv_carry_kernel(const float* __restrict__ proj, int width, int off, int C, int taps, float* __restrict__ conv_state,
+                      long long stride, const int* __restrict__ cu_seqlens, const int* __restrict__ slots) {
+  const int b = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int row0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - row0;
+  float* st = conv_state + (long long)slots[b] * stride;
+  float old[SSM_MAX_TAPS - 1];
+#pragma unroll
+  for (int s = 0; s < SSM_MAX_TAPS - 1; ++s) old[s] = s < taps - 1 ? st[(size_t)s * C + c] : 0.f;
+#pragma unroll
+  for (int s = 0; s < SSM_MAX_TAPS - 1; ++s) {
+    if (s >= taps - 1) break;
+    const int src = n_new - (taps - 1) + s;
+    float val = 0.f;
+    if (src >= 0) {
+      val = proj[(size_t)(row0 + src) * width + off + c];
+    } else {
+#pragma unroll
+      for (int q = 0; q < SSM_MAX_TAPS - 1; ++q)
+        if (q == s + n_new) val = old[q];
+    }
+    st[(size_t)s * C + c] = val;
+  }
+}
+
+// The recurrence, row after row: one workgroup per (head, sequence).  Thread (slice s, column d)
+// keeps rows s, s + nsl, ... of column d of the state in registers (R of them at most).
+template <typename T, int R>
+__global__ void __launch_bounds__(256)
+ssm_scan_kernel(const T* __restrict__ u, int C, int inner, int G, int N, int heads, int dv, const float* __restrict__ proj,
+                int width, int dt_off, const float* __restrict__ dt_bias, const float* __restrict__ A_log,
+                const float* __restrict__ Dw, float* __restrict__ state, long long stride, const int* __restrict__ cu_seqlens,
+                const int* __restrict__ slots, float* __restrict__ y) {
+  __shared__ float xs[SSM_TB][SSM_MAX_DV], Bs[SSM_TB][SSM_MAX_N], Cs[SSM_TB][SSM_MAX_N];
+  __shared__ float as[SSM_TB], dts[SSM_TB];
+  __shared__ float part[2][256];
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int g = h / (heads / G);
+  const int t = threadIdx.x;
+  const int nsl = 256 / dv;
+  const bool active = t < nsl * dv;
+  const int d = t % dv, s = t / dv;
+  const int row0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - row0;
+  float* S_g = state + (long long)slots[b] * stride + (size_t)h * N * dv;
+  float S[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int nr = s + r * nsl;
+    S[r] = (active && nr < N) ? S_g[(size_t)nr * dv + d] : 0.f;
+  }
+  const float neg_rate = -expf(A_log[h]);
+  const float bias = dt_bias[h], skip = Dw[h];
+  int parity = 0;
+  for (int i0 = 0; i0 < n_new; i0 += SSM_TB) {
+    const int tb = min(SSM_TB, n_new - i0);
+    __syncthreads();                     // the last batch's rows have been read
+    for (int e = t; e < tb * dv; e += 256) xs[e / dv][e % dv] = to_f32(u[(size_t)(row0 + i0 + e / dv) * C + h * dv + e % dv]);
+    for (int e = t; e < tb * N; e += 256) {
+      const size_t at = (size_t)(row0 + i0 + e / N) * C + inner + g * N + e % N;
+      Bs[e / N][e % N] = to_f32(u[at]);
+      Cs[e / N][e % N] = to_f32(u[at + (size_t)G * N]);
+    }
+    if (t < tb) {
+      const float dt = softplus_f(proj[(size_t)(row0 + i0 + t) * width + dt_off + h] + bias);
+      dts[t] = dt;
+      as[t] = expf(neg_rate * dt);
+    }
+    __syncthreads();
+    for (int i = 0; i < tb; ++i) {
+      const float a = as[i], dt = dts[i];
+      const float x = active ? xs[i][d] : 0.f;
+      const float dtx = dt * x;
+      float acc = 0.f;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int nr = s + r * nsl;
+        if (nr < N) {
+          S[r] = fmaf(a, S[r], Bs[i][nr] * dtx);
+          acc = fmaf(S[r], Cs[i][nr], acc);
+        }
+      }
+      part[parity][t] = acc;
+      __syncthreads();
+      if (t < dv) {
+        float sum = 0.f;
+        for (int q = 0; q < nsl; ++q) sum += part[parity][q * dv + t];
+        y[(size_t)(row0 + i0 + i) * inner + h * dv + t] = fmaf(skip, xs[i][t], sum);
+      }
+      parity ^= 1;
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int nr = s + r * nsl;
+    if (active && nr < N) S_g[(size_t)nr * dv + d] = S[r];
+  }
+}
+
+// out[n, part] = rms(y * silu(z)) * w over each of `parts` equal parts of the row.
+template <typename T>
+__global__ void __launch_bounds__(256)
+ssm_gate_norm_kernel(const float* __restrict__ y, const float* __restrict__ proj, int width, int inner, int parts,
+                     const float* __restrict__ w, float eps, T* __restrict__ out) {
+  __shared__ float sh[4];
+  const int n = blockIdx.x, part = blockIdx.y;
+  const int P = inner / parts;
+  const float* yr = y + (size_t)n * inner + part * P;
+  const float* zr = proj + (size_t)n * width + part * P;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < P; i += 256) {
+    const float a = yr[i] * silu_f(zr[i]);
+    ss += a * a;
+  }
+  ss = block_sum<256>(ss, sh);
+  const float f = 1.0f / sqrtf(ss / (float)P + eps);
+  for (int i = threadIdx.x; i < P; i += 256) {
+    const float a = yr[i] * silu_f(zr[i]);
+    out[(size_t)n * inner + part * P + i] = from_f32<T>(a * f * w[part * P + i]);
+  }
+}
+
+}  // namespace tl
+
+using namespace tl;
+
+template <typename T>
+static int scan_launch(int R, dim3 grid, hipStream_t st, const T* u, int C, int inner, int G, int N, int heads, int dv,
+                       const float* proj, int width, int dt_off, const float* dt_bias, const float* A_log, const float* D,
+                       float* state, long long stride, const int* cu, const int* slots, float* y) {
+#define TL_SCAN(RR)                                                                                                     \
+  ssm_scan_kernel<T, RR><<<grid, 256, 0, st>>>(u, C, inner, G, N, heads, dv, proj, width, dt_off, dt_bias, A_log, D, state, \
+                                               stride, cu, slots, y)
+  if (R <= 8) TL_SCAN(8);
+  else if (R <= 16) TL_SCAN(16);
+  else if (R <= 32) TL_SCAN(32);
+  else TL_SCAN(64);
+#undef TL_SCAN
+  return 0;
+}
+
+extern "C" {
+
+// proj [n, width]: the convolution's input are its columns off .. off + C - 1.
+int tl_ssm_conv(const float* proj, int width, int off, int C, const float* w, const float* bias, int taps,
+                float* conv_state, long long stride, const int* row_seq, const int* cu_seqlens, const int* slots, int n,
+                int B, void* out, int dt, hipStream_t st) {
+  TL_REQUIRE(n >= 0 && B >= 0 && C > 0 && off >= 0 && off + C <= width, "ssm_conv: bad sizes n=%d C=%d off=%d width=%d", n, C,
+             off, width);
+  TL_REQUIRE(taps >= 1 && taps <= SSM_MAX_TAPS, "ssm_conv: %d taps (1..%d)", taps, SSM_MAX_TAPS);
+  TL_REQUIRE(proj && w && conv_state && row_seq && cu_seqlens && slots && out, "ssm_conv: a buffer is missing");
+  TL_REQUIRE(stride >= (long long)(taps - 1) * C, "ssm_conv: a sequence's block is too small for %d rows of %d", taps - 1, C);
+  TL_REQUIRE(dt == DT_F32 || dt == DT_BF16, "ssm_conv: unknown dtype code %d", dt);
+  if (n == 0 || B == 0) return 0;
+  const dim3 grid(n, (C + 255) / 256);
+  if (dt == DT_F32)
+    ssm_conv_kernel<float><<<grid, 256, 0, st>>>(proj, width, off, C, w, bias, taps, conv_state, stride, row_seq, cu_seqlens,
+                                                 slots, (float*)out);
+  else
+    ssm_conv_kernel<bf16><<<grid, 256, 0, st>>>(proj, width, off, C, w, bias, taps, conv_state, stride, row_seq, cu_seqlens,
+                                                slots, (bf16*)out);
+  TL_LAUNCH_CHECK("ssm_conv");
+  if (taps > 1) {
+    ssm_conv_carry_kernel<<<dim3(B, (C + 255) / 256), 256, 0, st>>>(proj, width, off, C, taps, conv_state, stride, cu_seqlens,
+                                                                     slots);
+    TL_LAUNCH_CHECK("ssm_conv_carry");
+  }
+  return 0;
+}
+
+// u [n, C] = [x | B | C] after the convolution; proj [n, width] holds dt at column dt_off + h.
+int tl_ssm_scan(const void* u, int dt, int C, int G, int N, int heads, int dv, const float* proj, int width, int dt_off,
+                const float* dt_bias, const float* A_log, const float* D, float* state, long long stride,
+                const int* cu_seqlens, const int* slots, int n, int B, float* y, hipStream_t st) {
+  TL_REQUIRE(n >= 0 && B >= 0 && heads > 0 && G > 0 && heads % G == 0 && N > 0 && dv > 0, "ssm_scan: bad sizes heads=%d G=%d N=%d dv=%d",
+             heads, G, N, dv);
+  TL_REQUIRE(N <= SSM_MAX_N && dv <= SSM_MAX_DV, "ssm_scan: a state of %d x %d is not served (up to %d x %d)", N, dv, SSM_MAX_N,
+             SSM_MAX_DV);
+  const int inner = heads * dv;
+  TL_REQUIRE(C == inner + 2 * G * N && dt_off >= 0 && dt_off + heads <= width, "ssm_scan: %d channels for heads=%d dv=%d G=%d N=%d", C,
+             heads, dv, G, N);
+  const int nsl = 256 / dv, R = (N + nsl - 1) / nsl;
+  TL_REQUIRE(R <= 64, "ssm_scan: a state of %d x %d gives a thread %d rows (at most 64)", N, dv, R);
+  TL_REQUIRE(stride >= (long long)heads * N * dv, "ssm_scan: a sequence's block is too small");
+  TL_REQUIRE(u && proj && dt_bias && A_log && D && state && cu_seqlens && slots && y, "ssm_scan: a buffer is missing");
+  TL_REQUIRE(dt == DT_F32 || dt == DT_BF16, "ssm_scan: unknown dtype code %d", dt);
+  if (n == 0 || B == 0) return 0;
+  const dim3 grid(heads, B);
+  if (dt == DT_F32)
+    scan_launch<float>(R, grid, st, (const float*)u, C, inner, G, N, heads, dv, proj, width, dt_off, dt_bias, A_log, D, state, stride,
+                       cu_seqlens, slots, y);
+  else
+    scan_launch<bf16>(R, grid, st, (const bf16*)u, C, inner, G, N, heads, dv, proj, width, dt_off, dt_bias, A_log, D, state, stride,
+                      cu_seqlens, slots, y);
+  TL_LAUNCH_CHECK("ssm_scan");
+  return 0;
+}
+
+// y [n, inner] float, z = the first `inner` columns of proj [n, width].
+int tl_ssm_gate_norm(const float* y, const float* proj, int width, int inner, int parts, const float* w, float eps, int n,
+                     void* out, int dt, hipStream_t st) {
+  TL_REQUIRE(n >= 0 && inner > 0 && parts > 0 && inner % parts == 0 && inner <= width, "ssm_gate_norm: bad sizes inner=%d parts=%d width=%d",
+             inner, parts, width);
+  TL_REQUIRE(y && proj && w && out, "ssm_gate_norm: a buffer is missing");
+  TL_REQUIRE(dt == DT_F32 || dt == DT_BF16, "ssm_gate_norm: unknown dtype code %d", dt);
+  if (n == 0) return 0;
+  const dim3 grid(n, parts);
+  if (dt == DT_F32)
+    ssm_gate_norm_kernel<float><<<grid, 256, 0, st>>>(y, proj, width, inner, parts, w, eps, (float*)out);
+  else
+    ssm_gate_norm_kernel<bf16><<<grid, 256, 0, st>>>(y, proj, width, inner, parts, w, eps, (bf16*)out);
+  TL_LAUNCH_CHECK("ssm_gate_norm");
+  return 0;
+}
+
+}  // extern "C"

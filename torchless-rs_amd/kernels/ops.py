@@ -377,7 +377,7 @@ def cast_rows(x: torch.Tensor, out: torch.Tensor) -> None:
 # The functions of a gated feed-forward.  silu: g / (1 + e^-g); gelu_tanh: the tanh form of gelu;
 # swish_clamped, with the constants `alpha`, `limit` and `shift`: g' = min(g, limit),
 # u' = clamp(u, -limit, limit), and the hidden value is g' / (1 + e^(-alpha g')) * (u' + shift).
-ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "swish_clamped": 2}
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "swish_clamped": 2, "relu": 3}
 ACTIVATION_CONSTANTS = {"swish_clamped": ("alpha", "limit", "shift")}
 
 
@@ -404,11 +404,14 @@ def act_mul(gu: torch.Tensor, out: torch.Tensor, activation: str = "silu", const
 class ScoreTerms:
     """What an attention adds to q.k * scale: `slopes` (float32 [nq] or None), a bias
     -slope[h] * (p - j) by the distance of query and key; `sinks` (float32 [nq] or None), a score
-    per head with no key and no value that takes part in the softmax's sum once; `window`."""
+    per head with no key and no value that takes part in the softmax's sum once; `window`;
+    `keep_first`: with a window, the first positions of a sequence that stay visible beside it
+    (the cache must then keep every position: a ring would overwrite them)."""
 
     def __init__(self, scale: float, window: Optional[int] = None, slopes: Optional[torch.Tensor] = None,
-                 sinks: Optional[torch.Tensor] = None):
+                 sinks: Optional[torch.Tensor] = None, keep_first: int = 0):
         self.scale, self.window, self.slopes, self.sinks = float(scale), (int(window) if window else None), slopes, sinks
+        self.keep_first = int(keep_first) if self.window else 0
 
 
 def _req_pages(pages: torch.Tensor, nkv: int, dk: int, dv: int, what: str) -> None:
@@ -448,7 +451,7 @@ def attn_scored_plain(q, k_new, v_new, pages, nkv: int, dv: int, table, ring_pag
         raise KernelError("attn_scored.table: needs one row per sequence")
     _check(lib().tl_attn_scored_plain(_p(q), _p(k_new), _p(v_new), _p(pages), _code(q.dtype), _p(table),
                                       table.shape[1], ring_pages, _p(row_seq), _p(row_pos), _p(cu_seqlens),
-                                      _p(n_cached), n, nq, nkv, dk, dv, int(terms.window or 0),
+                                      _p(n_cached), n, nq, nkv, dk, dv, int(terms.window or 0), terms.keep_first,
                                       ctypes.c_float(terms.scale), _p(terms.slopes), _p(terms.sinks), _p(gate),
                                       _p(out), _code(out.dtype), _stream()))
 
@@ -457,6 +460,11 @@ def scored_on_matrix_cores(dtype: torch.dtype, dk: int, dv: int) -> bool:
     """Does `attention_scored` run on the matrix cores (bfloat16, values as wide as keys, head sizes in
     steps of 16)?  Steps with several rows a sequence then take their values transposed (`vt_new`)."""
     return dtype == torch.bfloat16 and dk == dv and dk % 16 == 0 and 16 <= dk <= 256
+
+
+def terms_on_matrix_cores(terms: ScoreTerms) -> bool:
+    """Do the matrix-core kernels know every term of `terms`?"""
+    return not terms.keep_first
 
 
 def _terms_args(terms: ScoreTerms, gate, n: int, nq: int):
@@ -477,7 +485,7 @@ def attention_scored(q, k_new, v_new, pages, nkv: int, dv: int, table, ring_page
     in the TERMS variant of the kernels of `attention` (the latter takes the step's values
     transposed, `vt_new`); everything else in the plain kernel."""
     n, nq, dk = q.shape
-    fast = scored_on_matrix_cores(q.dtype, dk, dv) and pages.dim() == 5
+    fast = scored_on_matrix_cores(q.dtype, dk, dv) and pages.dim() == 5 and terms_on_matrix_cores(terms)
     if fast and k_new is None and ctx.all_single:
         splits = decode_splits(n, nq, nkv, table.shape[1], compute_units(q.device), dk)
         part = ctx.workspace.get("attn_part", (n * nq * splits * (dk + 2),), torch.float32)
@@ -663,6 +671,158 @@ def diff_combine(att: torch.Tensor, lam: float, eps: float, post: float, out: to
                                  ctypes.c_float(post), _p(out), _code(out.dtype), _stream()))
 
 
+class HeadTerms:
+    """What happens to a row of the fused projection [q | k | v | g] of an attention before the
+    attention itself, head by head (`head_prepare`): `bias` (float32 over the whole row, or None);
+    `q_norm`, `k_norm` (float32 [dk] each, or None): every head divided by its own root mean
+    square (eps inside the root) times a weight that all heads share; `mix`: 0, or 1 (the values
+    are left, unrounded, for later layers) or 2 (v <- (1 - lam) v + lam * the values that were left)."""
+
+    def __init__(self, bias=None, q_norm=None, k_norm=None, eps: float = 0.0, mix: int = 0, lam: float = 0.0):
+        self.bias, self.q_norm, self.k_norm, self.eps = bias, q_norm, k_norm, float(eps)
+        self.mix, self.lam = int(mix), float(lam)
+
+
+def head_prepare(proj: torch.Tensor, row_pos, rotation, terms: HeadTerms, nq: int, nkv: int, dk: int, dv: int, ng: int,
+                 q: torch.Tensor, k, v, gate, v_first=None, table=None, ring_pages: int = 0, pages=None) -> None:
+    """proj float32 [n, nq*dk + nkv*(dk+dv) + ng] -> q [n, nq, dk] (biased, normed per head, rotated),
+    `gate` float32 [n, ng] (after the logistic function) and k [n, nkv, dk] and v [n, nkv, dv], or,
+    with `pages` (one token a sequence, row n belongs to sequence n), k and v straight into the
+    page of the row's position.  `v_first` (float32 [n, nkv*dv]): where a layer that mixes values
+    leaves or finds the first such layer's."""
+    n = proj.shape[0]
+    width = nq * dk + nkv * (dk + dv) + ng
+    rot = _rotation(rotation, dk, "head_prepare")
+    if rot.interleaved:
+        raise KernelError("head_prepare: pairs (2i, 2i + 1) are not served, only (i, i + rotary_dim / 2)")
+    _req(proj, "head_prepare.proj", torch.float32, (n, width))
+    _req(row_pos, "head_prepare.row_pos", torch.int32, (n,))
+    _req(q, "head_prepare.q", None, (n, nq, dk))
+    for t, name, size in ((terms.bias, "bias", width), (terms.q_norm, "q_norm", dk), (terms.k_norm, "k_norm", dk)):
+        if t is not None:
+            _req(t, "head_prepare." + name, torch.float32, (size,))
+    if ng:
+        _req(gate, "head_prepare.gate", torch.float32, (n, ng))
+    if terms.mix:
+        if v_first is None:
+            raise KernelError("head_prepare: mixing values needs the buffer they are left in")
+        _req(v_first, "head_prepare.v_first", torch.float32, (n, nkv * dv))
+    stride = 0
+    if pages is None:
+        _req(k, "head_prepare.k", q.dtype, (n, nkv, dk))
+        _req(v, "head_prepare.v", q.dtype, (n, nkv, dv))
+    else:
+        _req_pages(pages, nkv, dk, dv, "head_prepare")
+        _req(table, "head_prepare.table", torch.int32)
+        if pages.dtype != q.dtype or table.dim() != 2 or table.shape[0] != n:
+            raise KernelError("head_prepare: pages of q's dtype and a page table with one row per row")
+        stride = table.shape[1]
+    _check(lib().tl_head_prepare(_p(proj), _p(row_pos), _p(rot.inv_freq), rot.rotary_dim, _p(terms.bias), _p(terms.q_norm),
+                                 _p(terms.k_norm), ctypes.c_float(terms.eps), terms.mix, ctypes.c_float(terms.lam),
+                                 _p(v_first) if terms.mix else None, n, nq, nkv, dk, dv, ng, _p(q),
+                                 _p(k) if pages is None else None, _p(v) if pages is None else None, _p(gate),
+                                 _code(q.dtype), _p(table), stride, int(ring_pages), _p(pages), _stream()))
+
+
+# ---- the state-space mixer ---------------------------------------------------------------------------
+def ssm_conv(proj: torch.Tensor, off: int, C: int, w: torch.Tensor, bias, conv_state: torch.Tensor, row_seq, cu_seqlens,
+             slots, out: torch.Tensor) -> None:
+    """The short causal convolution of a state-space mixer over the columns off .. off + C - 1 of proj
+    (float32 [n, width]) and silu: out[n, c] = silu(bias[c] + sum_j w[c, j] * u[row - (taps - 1 - j), c]).  Rows
+    before the step come from the sequence's block `conv_state` [slots, >= (taps - 1) * C] (float32, the
+    oldest row first, zeros before the start), which afterwards holds the step's last taps - 1 inputs."""
+    n, width = proj.shape
+    taps = w.shape[1]
+    B = slots.shape[0]
+    _req(proj, "ssm_conv.proj", torch.float32)
+    _req(w, "ssm_conv.w", torch.float32, (C, taps))
+    if bias is not None:
+        _req(bias, "ssm_conv.bias", torch.float32, (C,))
+    if conv_state.dtype != torch.float32 or conv_state.dim() != 2 or conv_state.stride(1) != 1 or not conv_state.is_cuda:
+        raise KernelError("ssm_conv.conv_state: float32 [slots, block] on the GPU, rows may be strided")
+    _req(row_seq, "ssm_conv.row_seq", torch.int32, (n,))
+    _req(cu_seqlens, "ssm_conv.cu_seqlens", torch.int32, (B + 1,))
+    _req(slots, "ssm_conv.slots", torch.int32)
+    _req(out, "ssm_conv.out", None, (n, C))
+    if conv_state.shape[1] < (taps - 1) * C:
+        raise KernelError(f"ssm_conv: a block of {conv_state.shape[1]} for {taps - 1} rows of {C}")
+    _check(lib().tl_ssm_conv(_p(proj), width, int(off), int(C), _p(w), _p(bias), taps, _p(conv_state),
+                             ctypes.c_longlong(conv_state.stride(0)), _p(row_seq), _p(cu_seqlens), _p(slots), n, B, _p(out),
+                             _code(out.dtype), _stream()))
+
+
+def ssm_scan(u: torch.Tensor, proj: torch.Tensor, dt_off: int, G: int, N: int, heads: int, dv: int, dt_bias, A_log, D,
+             state: torch.Tensor, cu_seqlens, slots, y: torch.Tensor) -> None:
+    """The recurrence of a state-space mixer over the rows of a step, sequence by sequence: u [n, heads*dv + 2*G*N]
+    = [x | B | C] (after the convolution), dt at the columns dt_off .. of proj (float32 [n, width]);
+    dt' = softplus(dt + dt_bias[h]), S <- exp(-exp(A_log[h]) dt') S + dt' B x^T, y = S^T C + D[h] x; `state`
+    float32 [slots, >= heads*N*dv] is read and left updated; y float32 [n, heads*dv]."""
+    n, C = u.shape
+    B = slots.shape[0]
+    _req(u, "ssm_scan.u")
+    _req(proj, "ssm_scan.proj", torch.float32)
+    for t, name in ((dt_bias, "dt_bias"), (A_log, "A_log"), (D, "D")):
+        _req(t, "ssm_scan." + name, torch.float32, (heads,))
+    if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or not state.is_cuda:
+        raise KernelError("ssm_scan.state: float32 [slots, block] on the GPU, rows may be strided")
+    if state.shape[1] < heads * N * dv or proj.shape[0] != n:
+        raise KernelError(f"ssm_scan: a block of {state.shape[1]} for a state of {heads} x {N} x {dv}")
+    _req(cu_seqlens, "ssm_scan.cu_seqlens", torch.int32, (B + 1,))
+    _req(slots, "ssm_scan.slots", torch.int32)
+    _req(y, "ssm_scan.y", torch.float32, (n, heads * dv))
+    _check(lib().tl_ssm_scan(_p(u), _code(u.dtype), C, G, N, heads, dv, _p(proj), proj.shape[1], int(dt_off), _p(dt_bias),
+                             _p(A_log), _p(D), _p(state), ctypes.c_longlong(state.stride(0)), _p(cu_seqlens), _p(slots), n, B,
+                             _p(y), _stream()))
+
+
+def ssm_gate_norm(y: torch.Tensor, proj: torch.Tensor, parts: int, w: torch.Tensor, eps: float, out: torch.Tensor) -> None:
+    """out = rms(y * silu(z)) * w over each of `parts` equal parts of a row; y float32 [n, inner], z the first
+    `inner` columns of proj (float32 [n, width]), w float32 [inner]."""
+    n, inner = y.shape
+    _req(y, "ssm_gate_norm.y", torch.float32)
+    _req(proj, "ssm_gate_norm.proj", torch.float32)
+    _req(w, "ssm_gate_norm.w", torch.float32, (inner,))
+    _req(out, "ssm_gate_norm.out", None, (n, inner))
+    if proj.shape[0] != n:
+        raise KernelError("ssm_gate_norm: y and proj differ in rows")
+    _check(lib().tl_ssm_gate_norm(_p(y), _p(proj), proj.shape[1], inner, int(parts), _p(w), ctypes.c_float(eps), n, _p(out),
+                                  _code(out.dtype), _stream()))
+
+
+# ---- routed experts ----------------------------------------------------------------------------------
+EXPERT_ACTIVATIONS = {"relu2": 0, "relu": 1}
+
+
+def route(h: torch.Tensor, router: torch.Tensor, groups: int, keep: int, top: int, weights: torch.Tensor,
+          chosen: Optional[torch.Tensor] = None) -> None:
+    """The router of a mixture of experts, in float32: s = softmax(router h) over the E experts; of the `keep`
+    groups (of `groups` equal groups of neighbours; 0: no groups) whose best s is largest, the `top` experts
+    with the largest s; `weights` float32 [n, E] receives s for those and 0 for the others, `chosen` (int32
+    [n, top], or None) their indices, the best first."""
+    n, W = h.shape
+    E = router.shape[0]
+    _req(h, "route.h")
+    _req(router, "route.router", torch.float32, (E, W))
+    _req(weights, "route.weights", torch.float32, (n, E))
+    if chosen is not None:
+        _req(chosen, "route.chosen", torch.int32, (n, top))
+    _check(lib().tl_route(_p(h), _code(h.dtype), n, W, _p(router), E, int(groups), int(keep), int(top), _p(weights),
+                          _p(chosen), _stream()))
+
+
+def expert_act(u: torch.Tensor, weights: Optional[torch.Tensor], E: int, ff: int, activation: str, out: torch.Tensor) -> None:
+    """out[n, j] = act(u[n, j]) * (weights[n, j // ff] for the first E * ff columns, 1 for the rest); u float32."""
+    n, total = u.shape
+    if activation not in EXPERT_ACTIVATIONS:
+        raise KernelError(f"expert_act: no function {activation!r}; there are {sorted(EXPERT_ACTIVATIONS)}")
+    _req(u, "expert_act.u", torch.float32)
+    if E:
+        _req(weights, "expert_act.weights", torch.float32, (n, E))
+    _req(out, "expert_act.out", None, (n, total))
+    _check(lib().tl_expert_act(_p(u), _p(weights) if E else None, n, int(E), int(ff), total, EXPERT_ACTIVATIONS[activation],
+                               _p(out), _code(out.dtype), _stream()))
+
+
 def take_tokens(src: torch.Tensor, idx: torch.Tensor, vocab: int, tokens: torch.Tensor) -> None:
     """tokens[j] = src[idx[j]] (int32, on the device); ids outside [0, vocab) become 0."""
     n = tokens.shape[0]
@@ -709,7 +869,9 @@ EPI_STORE, EPI_ACCUMULATE, EPI_SILU_PAIR, EPI_GELU_PAIR = 0, 1, 2, 3
 
 
 EPI_SWISH_CLAMPED_PAIR = 4
-PAIR_EPILOGUES = {"silu": EPI_SILU_PAIR, "gelu_tanh": EPI_GELU_PAIR, "swish_clamped": EPI_SWISH_CLAMPED_PAIR}
+EPI_RELU_PAIR = 5
+PAIR_EPILOGUES = {"silu": EPI_SILU_PAIR, "gelu_tanh": EPI_GELU_PAIR, "swish_clamped": EPI_SWISH_CLAMPED_PAIR,
+                  "relu": EPI_RELU_PAIR}
 
 
 def _pair_epilogue(pair_act, constants=None) -> int:

@@ -6,6 +6,7 @@ from .. import parts as _parts            # registers the parts
 from . import mistral as _mistral         # registers MistralForCausalLM
 from . import sozetar as _sozetar         # registers Sozetar
 from . import fanitar as _fanitar         # registers Fanitar
+from . import nepisun as _nepisun         # registers Nepisun
 
 
 def model_spec_for(cfg: ModelConfig):

@@ -18,38 +18,45 @@ from .base import (LayerSpec, Part, expect_norm, flush_pending, make_part, part_
 
 
 class PreNormBlock(Part):
+    """x += mixer(norm(x)); then, if the layer has a feed-forward, x += ffn(norm(x))."""
+
     def __init__(self, layer: LayerSpec, mixer_norm_name: str = "input_layernorm.",
                  ffn_norm_name: str = "post_attention_layernorm."):
         self.mixer = make_part("mixer", layer.mixer)
-        self.ffn = make_part("ffn", layer.ffn)
+        self.ffn = make_part("ffn", layer.ffn) if layer.ffn is not None else None
         self.mixer_norm = make_part("norm", layer.mixer_norm)
-        self.ffn_norm = make_part("norm", layer.ffn_norm)
+        self.ffn_norm = make_part("norm", layer.ffn_norm) if layer.ffn is not None else None
         self.n1, self.n2 = mixer_norm_name, ffn_norm_name
-        self.graph_safe = all(p.graph_safe for p in (self.mixer, self.ffn, self.mixer_norm, self.ffn_norm))
+        self.graph_safe = all(p.graph_safe for p in self._parts())
+
+    def _parts(self):
+        return [p for p in (self.mixer, self.ffn, self.mixer_norm, self.ffn_norm) if p is not None]
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
         out: Dict[str, WeightSpec] = {}
         for k, v in self.mixer_norm.weight_specs().items():
             out[self.n1 + k] = v
         out.update(self.mixer.weight_specs())
-        for k, v in self.ffn_norm.weight_specs().items():
-            out[self.n2 + k] = v
-        out.update(self.ffn.weight_specs())
+        if self.ffn is not None:
+            for k, v in self.ffn_norm.weight_specs().items():
+                out[self.n2 + k] = v
+            out.update(self.ffn.weight_specs())
         return out
 
     def load(self, tensors, compute_dtype) -> None:
         def sub(prefix):
             return {k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)}
         self.mixer_norm.load(sub(self.n1), compute_dtype)
-        self.ffn_norm.load(sub(self.n2), compute_dtype)
         self.mixer.load(tensors, compute_dtype)
-        self.ffn.load(tensors, compute_dtype)
+        if self.ffn is not None:
+            self.ffn_norm.load(sub(self.n2), compute_dtype)
+            self.ffn.load(tensors, compute_dtype)
 
     def may_capture(self, n_rows: int) -> bool:
-        return all(p.may_capture(n_rows) for p in (self.mixer, self.ffn, self.mixer_norm, self.ffn_norm))
+        return all(p.may_capture(n_rows) for p in self._parts())
 
     def prefers_eager(self, n_new, len_before, device) -> bool:
-        return any(p.prefers_eager(n_new, len_before, device) for p in (self.mixer, self.ffn, self.mixer_norm, self.ffn_norm))
+        return any(p.prefers_eager(n_new, len_before, device) for p in self._parts())
 
     def entry_norm(self):
         """The norm that reads the stream first, if the part behind it can take a norm cut in
@@ -63,9 +70,14 @@ class PreNormBlock(Part):
         ctx.host.pop("stream_copy", None)        # this block writes the stream: a copy of it goes stale
         y = ctx.workspace.get("block_y", tuple(x.shape), ctx.dtype)
         y1 = read_through_norm(ctx, self.mixer_norm, x, y)
-        expect_norm(ctx, self.mixer, self.ffn_norm, self.ffn)
+        if self.ffn is None:
+            expect_norm(ctx, self.mixer, norm_after)
+        else:
+            expect_norm(ctx, self.mixer, self.ffn_norm, self.ffn)
         self.mixer.forward(ctx, run, y1, x)
         part_done(ctx, self.mixer)
+        if self.ffn is None:
+            return
         y2 = read_through_norm(ctx, self.ffn_norm, x, y)
         expect_norm(ctx, self.ffn, norm_after)
         self.ffn.forward(ctx, y2, x)

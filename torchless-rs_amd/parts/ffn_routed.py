@@ -1,0 +1,146 @@
+"""Feed-forwards without a gate, and a routed mixture of them.
+
+`PlainFeedForward`: down(act(up y)), act one of `ops.EXPERT_ACTIVATIONS` (relu2: the square of
+max(., 0)).
+
+`RoutedExperts`: `n_experts` such layers of which every token uses `top`.  The router is one
+more product, in float32: s = softmax(W_r y) over all experts.  The experts form
+`group_count` equal groups of neighbours; a group's score is its largest s, and only experts of
+the `group_keep` best groups can be chosen (no groups: any expert).  The `top` experts with the
+largest s are chosen; the result is the sum of their outputs weighted by their s, not
+renormalised, plus a shared expert's (`shared_size`; None: none) that runs for every token.
+
+All experts run as ONE wide feed-forward: their up projections stacked by rows (the shared
+expert's behind them), the activation times the row's weight of the column's expert, which is
+zero for an expert that was not chosen, and their down projections side by side.  That is two
+products of the framework's own kinds and no gather or scatter, whatever the tokens choose; it
+reads every expert's weights in every step, as a step of several sequences does anyway, and
+multiplies `n_experts / top` times what the chosen experts alone would.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..kernels import ops
+from ..weights.binding import WeightSpec
+from .base import FeedForward, register_part
+from .linear import Linear
+
+
+class PlainFeedForward(FeedForward):
+    graph_safe = True
+    closes_stream = True
+
+    NAMES = {"up": "up", "down": "down"}
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "relu2", prefix: str = "mlp.",
+                 names: Optional[Dict[str, str]] = None):
+        if activation not in ops.EXPERT_ACTIVATIONS:
+            raise ValueError(f"feed-forward: no activation {activation!r}; there are {sorted(ops.EXPERT_ACTIVATIONS)}")
+        self.H, self.I, self.activation, self.prefix = int(hidden_size), int(intermediate_size), activation, prefix
+        self.names = dict(self.NAMES, **(names or {}))
+        self.up = self.down = None
+
+    def may_capture(self, n_rows: int) -> bool:
+        return self.up is not None and self.up.own_kernels(n_rows) and self.down.own_kernels(n_rows)
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        p, nm = self.prefix, self.names
+        return {p + nm["up"]: WeightSpec((self.I, self.H)), p + nm["down"]: WeightSpec((self.H, self.I))}
+
+    def load(self, tensors, compute_dtype) -> None:
+        p, nm = self.prefix, self.names
+        self.up = Linear(tensors[p + nm["up"]], tiled=True)
+        self.down = Linear(tensors[p + nm["down"]], tiled=True)
+
+    def _hidden(self, ctx, y: torch.Tensor) -> torch.Tensor:
+        n = y.shape[0]
+        u = ctx.workspace.get("pff_u", (n, self.I), torch.float32)
+        self.up(y, u)
+        h = ctx.workspace.get("pff_h", (n, self.I), ctx.dtype)
+        ops.expert_act(u, None, 0, self.I, self.activation, h)
+        return h
+
+    def forward(self, ctx, y: torch.Tensor, x: torch.Tensor) -> None:
+        self.down.add_into(self._hidden(ctx, y), x, ctx, "pff_down_parts")
+
+    def produce(self, ctx, y: torch.Tensor, out: torch.Tensor) -> None:
+        self.down(self._hidden(ctx, y), out)
+
+
+class RoutedExperts(FeedForward):
+    graph_safe = True
+    closes_stream = True
+
+    # leaf names under `prefix`; "{e}" is the expert's number
+    NAMES = {"router": "router", "up": "e{e}.up", "down": "e{e}.down", "shared_up": "shared.up",
+             "shared_down": "shared.down"}
+
+    def __init__(self, hidden_size: int, n_experts: int, top: int, expert_size: int, group_count: Optional[int] = None,
+                 group_keep: Optional[int] = None, shared_size: Optional[int] = None, activation: str = "relu2",
+                 prefix: str = "mlp.", names: Optional[Dict[str, str]] = None):
+        if activation not in ops.EXPERT_ACTIVATIONS:
+            raise ValueError(f"experts: no activation {activation!r}; there are {sorted(ops.EXPERT_ACTIVATIONS)}")
+        if not (1 <= top <= n_experts):
+            raise ValueError(f"experts: {top} of {n_experts}")
+        if group_count:
+            if n_experts % group_count or not (1 <= (group_keep or 0) <= group_count) or group_keep * (n_experts // group_count) < top:
+                raise ValueError(f"experts: {n_experts} in {group_count} groups of which {group_keep} are kept cannot give {top}")
+        self.H, self.E, self.top, self.ff = int(hidden_size), int(n_experts), int(top), int(expert_size)
+        self.groups, self.keep = (int(group_count), int(group_keep)) if group_count else (0, 0)
+        self.shared = int(shared_size) if shared_size else 0
+        self.total = self.E * self.ff + self.shared
+        self.activation, self.prefix = activation, prefix
+        self.names = dict(self.NAMES, **(names or {}))
+        self.router = self.up = self.down = None
+
+    def may_capture(self, n_rows: int) -> bool:
+        return self.up is not None and self.up.own_kernels(n_rows) and self.down.own_kernels(n_rows)
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        p, nm = self.prefix, self.names
+        out: Dict[str, WeightSpec] = {}
+        for e in range(self.E):
+            out[p + nm["up"].format(e=e)] = WeightSpec((self.ff, self.H))
+            out[p + nm["down"].format(e=e)] = WeightSpec((self.H, self.ff))
+        out[p + nm["router"]] = WeightSpec((self.E, self.H))
+        if self.shared:
+            out[p + nm["shared_up"]] = WeightSpec((self.shared, self.H))
+            out[p + nm["shared_down"]] = WeightSpec((self.H, self.shared))
+        return out
+
+    def load(self, tensors, compute_dtype) -> None:
+        p, nm = self.prefix, self.names
+        ups = [tensors[p + nm["up"].format(e=e)] for e in range(self.E)]
+        downs = [tensors[p + nm["down"].format(e=e)] for e in range(self.E)]
+        if self.shared:
+            ups.append(tensors[p + nm["shared_up"]])
+            downs.append(tensors[p + nm["shared_down"]])
+        if len({w.dtype for w in ups + downs}) > 1:
+            ups, downs = [w.to(torch.float32) for w in ups], [w.to(torch.float32) for w in downs]
+        self.up = Linear(torch.cat(ups, dim=0), tiled=True)          # [E * ff + shared, H]
+        self.down = Linear(torch.cat(downs, dim=1), tiled=True)      # [H, E * ff + shared]
+        self.router = tensors[p + nm["router"]].to(torch.float32).contiguous()
+
+    def _hidden(self, ctx, y: torch.Tensor) -> torch.Tensor:
+        n = y.shape[0]
+        ws = ctx.workspace
+        weights = ws.get("experts_w", (n, self.E), torch.float32)
+        ops.route(y, self.router, self.groups, self.keep, self.top, weights)
+        u = ws.get("experts_u", (n, self.total), torch.float32)
+        self.up(y, u)
+        h = ws.get("experts_h", (n, self.total), ctx.dtype)
+        ops.expert_act(u, weights, self.E, self.ff, self.activation, h)
+        return h
+
+    def forward(self, ctx, y: torch.Tensor, x: torch.Tensor) -> None:
+        self.down.add_into(self._hidden(ctx, y), x, ctx, "experts_down_parts")
+
+    def produce(self, ctx, y: torch.Tensor, out: torch.Tensor) -> None:
+        self.down(self._hidden(ctx, y), out)
+
+
+register_part("ffn", "plain", PlainFeedForward)
+register_part("ffn", "routed_experts", RoutedExperts)
