@@ -131,8 +131,33 @@ def causal_conv(u, weight, bias):
     return out
 
 
+def recurrence(xs, Bm, Cm, dt, A_log, D, S=None):
+    """xs [T, Hd, dv], Bm and Cm [T, G, N], dt [T, Hd] (after softplus): per head S <- exp(-exp(A) dt) S + dt B x^T,
+    y = S^T C + D x.  Returns (y [T, Hd, dv], the last S [Hd, N, dv])."""
+    T, Hd, dv = xs.shape
+    G, N = Bm.shape[1], Bm.shape[2]
+    per = Hd // G
+    decay = torch.exp(-torch.exp(A_log)[None, :] * dt)
+    S = torch.zeros(Hd, N, dv, dtype=xs.dtype) if S is None else S
+    ys = []
+    for t in range(T):
+        Bt = Bm[t].repeat_interleave(per, dim=0)             # [Hd, N]
+        Ct = Cm[t].repeat_interleave(per, dim=0)
+        S = decay[t][:, None, None] * S + dt[t][:, None, None] * Bt[:, :, None] * xs[t][:, None, :]
+        ys.append((S * Ct[:, :, None]).sum(dim=1) + D[:, None] * xs[t])
+    return torch.stack(ys), S
+
+
+def gated_group_norm(y, z, parts, eps, w):
+    """y * silu(z), normed in `parts` equal parts of the row, times w."""
+    T, inner = y.shape
+    g = y * silu(z)
+    return rms(g.view(T, parts, inner // parts), eps).reshape(T, inner) * w
+
+
 def state_space(h, w, p, m, eps):
-    """Kind `mamba2`: per head a state S [N, dv]: S <- exp(-exp(A) dt) S + dt B x^T, y = S^T C + D x."""
+    """Kind `mamba2`: one projection to [z | x B C | dt], a short causal convolution and silu on x B C,
+    the recurrence, the gated norm in parts, the output projection."""
     T = h.shape[0]
     Hd, dv, N, G = m["heads"], m["vdim"], m["state"], m["groups"]
     inner = Hd * dv
@@ -143,20 +168,8 @@ def state_space(h, w, p, m, eps):
     Bm = xbc[:, inner:inner + G * N].view(T, G, N)
     Cm = xbc[:, inner + G * N:].view(T, G, N)
     dt = torch.nn.functional.softplus(dt + w[p + "dt_bias"], threshold=1e9)       # [T, Hd]
-    decay = torch.exp(-torch.exp(w[p + "A_log"])[None, :] * dt)
-    per = Hd // G
-    S = torch.zeros(Hd, N, dv, dtype=h.dtype)
-    ys = []
-    for t in range(T):
-        Bt = Bm[t].repeat_interleave(per, dim=0)             # [Hd, N]
-        Ct = Cm[t].repeat_interleave(per, dim=0)
-        S = decay[t][:, None, None] * S + dt[t][:, None, None] * Bt[:, :, None] * xs[t][:, None, :]
-        y = (S * Ct[:, :, None]).sum(dim=1) + w[p + "D"][:, None] * xs[t]
-        ys.append(y.reshape(inner))
-    y = torch.stack(ys) * silu(z)
-    parts = m["norm_groups"]
-    y = rms(y.view(T, parts, inner // parts), eps).reshape(T, inner) * w[p + "norm"]
-    return y @ w[p + "o"].T
+    y, _ = recurrence(xs, Bm, Cm, dt, w[p + "A_log"], w[p + "D"])
+    return gated_group_norm(y.reshape(T, inner), z, m["norm_groups"], eps, w[p + "norm"]) @ w[p + "o"].T
 
 
 def dense_ff(h, w, p):
@@ -218,3 +231,87 @@ def forward(w, cfg, ids, dtype=F64, streams=None):
         if streams is not None:
             streams.append(x.clone())
     return rms(x, eps, w["final.norm"]) @ w["embed"].T
+
+
+def generate_greedy(w, cfg, ids, n, dtype=F64):
+    """n tokens, each the argmax of the last position's logits (of equal maxima the last)."""
+    ids, out = list(ids), []
+    for _ in range(n):
+        lg = forward(w, cfg, ids, dtype)[-1]
+        t = int((lg == lg.max()).nonzero().max())
+        out.append(t)
+        ids.append(t)
+    return out
+
+
+def tensor_shapes(cfg):
+    """Every tensor of a model of this configuration: name -> shape."""
+    W = cfg["width"]
+    out = {"embed": (cfg["vocab"], W), "final.norm": (W,)}
+    for i, layer in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", layer["mixer"]
+        out[p + "norm1"] = (W,)
+        if layer["type"] == "mamba2":
+            inner, GN = m["heads"] * m["vdim"], m["groups"] * m["state"]
+            C = inner + 2 * GN
+            out.update({p + "mix.in": (inner + C + m["heads"], W), p + "mix.conv": (C, m["conv"]), p + "mix.conv.b": (C,),
+                        p + "mix.dt_bias": (m["heads"],), p + "mix.A_log": (m["heads"],), p + "mix.D": (m["heads"],),
+                        p + "mix.norm": (inner,), p + "mix.o": (W, inner)})
+        else:
+            Q, K, V = m["heads"] * m["dim"], m["kv_heads"] * m["dim"], m["kv_heads"] * m["vdim"]
+            out.update({p + "mix.q": (Q, W), p + "mix.k": (K, W), p + "mix.v": (V, W), p + "mix.o": (W, m["heads"] * m["vdim"])})
+            if layer["type"] == "attention":
+                out.update({p + "mix.q.norm": (m["dim"],), p + "mix.k.norm": (m["dim"],), p + "mix.g": (m["heads"] * m["vdim"], W)})
+            else:
+                out.update({p + "mix.q.b": (Q,), p + "mix.k.b": (K,), p + "mix.v.b": (V,), p + "mix.o.b": (W,)})
+            if m.get("v_mix"):
+                out[p + "mix.vmix"] = ()
+        mlp = layer.get("mlp")
+        if not mlp:
+            continue
+        out[p + "norm2"] = (W,)
+        if mlp["kind"] == "dense":
+            out.update({p + "mlp.gate": (mlp["ff"], W), p + "mlp.up": (mlp["ff"], W), p + "mlp.down": (W, mlp["ff"])})
+        else:
+            for e in range(mlp["router"]["experts"]):
+                out[p + f"mlp.e{e}.up"] = (mlp["expert"]["ff"], W)
+                out[p + f"mlp.e{e}.down"] = (W, mlp["expert"]["ff"])
+            out[p + "mlp.router"] = (mlp["router"]["experts"], W)
+            if mlp.get("shared"):
+                out[p + "mlp.shared.up"] = (mlp["shared"]["ff"], W)
+                out[p + "mlp.shared.down"] = (W, mlp["shared"]["ff"])
+    return out
+
+
+def random_weights(cfg, seed, gain=1.0):
+    """bfloat16 tensors whose sizes follow the configuration, scaled so that every mechanism matters:
+    scores of a few units, router logits that differ, decays between 0.2 and 0.9, a mixing weight
+    well away from 0 and 1."""
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, shape in tensor_shapes(cfg).items():
+        leaf = name.split(".", 1)[1] if name.startswith("l") else name
+        if leaf in ("norm1", "norm2", "mix.norm") or name == "final.norm":
+            t = 1.0 + 0.2 * torch.randn(shape, generator=g)
+        elif leaf in ("mix.q.norm", "mix.k.norm"):
+            t = gain * (1.5 + 0.3 * torch.randn(shape, generator=g))
+        elif leaf == "mix.vmix":
+            t = torch.tensor(0.25 + 0.5 * float(torch.rand((), generator=g)))
+        elif leaf in ("mix.A_log", "mix.dt_bias"):
+            t = 0.6 * torch.randn(shape, generator=g)
+        elif leaf == "mix.D":
+            t = 1.0 + 0.3 * torch.randn(shape, generator=g)
+        elif leaf == "mix.conv":
+            t = torch.randn(shape, generator=g) * 0.6
+        elif leaf.endswith(".b"):
+            t = torch.randn(shape, generator=g) * 0.3
+        elif leaf == "mlp.router":
+            t = torch.randn(shape, generator=g) * (2.0 / shape[1] ** 0.5)
+        elif name == "embed":
+            t = torch.randn(shape, generator=g)
+        else:
+            t = torch.randn(shape, generator=g) * (1.0 / shape[1] ** 0.5)
+            if leaf in ("mix.q", "mix.k"):
+                t = t * gain
+        out[name] = t.to(torch.bfloat16)
+    return out
