@@ -180,24 +180,39 @@ def small_expert(h, w, p):
     return (torch.relu(h @ w[p + "up"].T) ** 2) @ w[p + "down"].T
 
 
-def route(h, w, p, r):
-    """The chosen experts of every token and their weights: [T, top] each."""
+def _gap(values, n):
+    """Per row, how far the n-th largest of `values` lies above the next one, as a share of itself (1 if there
+    is no next one)."""
+    if n >= values.shape[-1]:
+        return torch.ones(values.shape[0], dtype=values.dtype)
+    srt = values.sort(dim=-1, descending=True).values
+    return (srt[:, n - 1] - srt[:, n]) / srt[:, n - 1]
+
+
+def route(h, w, p, r, margins=None):
+    """The chosen experts of every token and their weights: [T, top] each.  `margins`, a list, receives per
+    token the smallest relative gap by which a group or an expert was chosen over the next one."""
     E, top = r["experts"], r["top"]
     s = torch.softmax(h @ w[p + "router"].T, dim=-1)                     # [T, E]
     allowed = torch.ones_like(s, dtype=torch.bool)
     groups = r.get("groups")
+    margin = torch.ones(s.shape[0], dtype=s.dtype)
     if groups:
         per = E // groups["count"]
         best = s.view(-1, groups["count"], per).max(dim=-1).values       # [T, count]
         kept = best.topk(groups["keep"], dim=-1).indices
         ok = torch.zeros_like(best, dtype=torch.bool).scatter_(1, kept, True)
         allowed = ok.repeat_interleave(per, dim=1)
+        margin = torch.minimum(margin, _gap(best, groups["keep"]))
+    masked = s.masked_fill(~allowed, 0.0)
     chosen = s.masked_fill(~allowed, -1.0).topk(top, dim=-1).indices
+    if margins is not None:
+        margins.append(torch.minimum(margin, _gap(masked, top)))
     return chosen, s.gather(1, chosen)
 
 
-def routed_ff(h, w, p, mlp):
-    chosen, weight = route(h, w, p, mlp["router"])
+def routed_ff(h, w, p, mlp, margins=None):
+    chosen, weight = route(h, w, p, mlp["router"], margins)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for e, g in zip(chosen[t].tolist(), weight[t]):
@@ -210,9 +225,10 @@ def routed_ff(h, w, p, mlp):
 MIXERS = {"attention": attention_gated, "attention_2": attention_windowed}
 
 
-def forward(w, cfg, ids, dtype=F64, streams=None):
+def forward(w, cfg, ids, dtype=F64, streams=None, margins=None):
     """Logits [T, V] of one prompt from the first position.  `streams`, a list, receives the
-    residual stream after every layer."""
+    residual stream after every layer; `margins`, a list, one tensor [T] per routed layer: by how
+    much the router's choice was made (see `route`)."""
     w = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in w.items()}
     eps = cfg["norm"]["eps"]
     x = w["embed"][torch.tensor(ids)]
@@ -227,7 +243,7 @@ def forward(w, cfg, ids, dtype=F64, streams=None):
         mlp = layer.get("mlp")
         if mlp:
             h = rms(x, eps, w[p + "norm2"])
-            x = x + (dense_ff(h, w, p + "mlp.") if mlp["kind"] == "dense" else routed_ff(h, w, p + "mlp.", mlp))
+            x = x + (dense_ff(h, w, p + "mlp.") if mlp["kind"] == "dense" else routed_ff(h, w, p + "mlp.", mlp, margins))
         if streams is not None:
             streams.append(x.clone())
     return rms(x, eps, w["final.norm"]) @ w["embed"].T
