@@ -111,6 +111,71 @@ def fanitar_counts(z: dict, layers: int, B: int, C: int, T: int):
     return w, kv, att
 
 
+def nepisun_layers(z: dict, layers: int):
+    """The layers of `nepisun_config(z, layers)` as (mixer kind, feed-forward kind): state-space layers and the two
+    kinds of attention in turn, the first feed-forward dense, the others routed."""
+    kinds = ["mamba2", "mamba2", "attention_2", "attention"]
+    return [(kinds[i % 4], "dense" if i % 4 == 0 else "moe") for i in range(layers)]
+
+
+def nepisun_sizes(z: dict):
+    """Sizes of the Nepisun layers at the layer sizes `z`: a state-space mixer of twice the width in heads of 64
+    with states of 128 rows; 16 experts of a quarter of the dense feed-forward's hidden size of which a token uses
+    4, beside a shared one of half of it: a token multiplies as much as in the dense feed-forward."""
+    return dict(ssm_heads=2 * z["width"] // 64, ssm_dv=64, state=128, groups=8, conv=4, experts=16, top=4,
+                expert_ff=z["ff"] // 4, shared_ff=z["ff"] // 2, keep_first=64)
+
+
+def nepisun_config(z: dict, layers: int):
+    """config.json of a Nepisun model with the layer sizes `z` (see `nepisun_layers`, `nepisun_sizes`)."""
+    n = nepisun_sizes(z)
+    out = []
+    for mix, ff in nepisun_layers(z, layers):
+        if mix == "mamba2":
+            m = {"heads": n["ssm_heads"], "vdim": n["ssm_dv"], "state": n["state"], "groups": n["groups"], "conv": n["conv"],
+                 "norm_groups": n["groups"]}
+        else:
+            m = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"], "scale": z["dim"] ** -0.5,
+                 "rot": {"base": 10000.0, "dims": z["dim"]}, "v_mix": True}
+            if mix == "attention_2" and z["window"]:
+                m["mask"] = {"size": z["window"], "keep_first": n["keep_first"]}
+        mlp = {"kind": "dense", "ff": z["ff"]} if ff == "dense" else {
+            "kind": "moe", "router": {"experts": n["experts"], "top": n["top"], "groups": {"count": 4, "keep": 2}},
+            "expert": {"ff": n["expert_ff"]}, "shared": {"ff": n["shared_ff"]}}
+        out.append({"type": mix, "mixer": m, "mlp": mlp})
+    return {"architecture": "Nepisun", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6}, "layers": out}
+
+
+def nepisun_counts(z: dict, layers: int, B: int, C: int, T: int):
+    """(weight elements that a prompt's products multiply a row by, bytes of keys, values and recurrent state that a
+    decode step reads and writes, multiply-adds times two of a prompt's attention and recurrence, weight elements that
+    a decode step of B rows must read) of `nepisun_config(z, layers)`.  A routed feed-forward multiplies a row by its
+    `top` experts and the shared one; a decode step reads the experts that B rows can choose at most."""
+    H, I, nq, nkv, d = z["width"], z["ff"], z["heads"], z["kv_heads"], z["dim"]
+    n = nepisun_sizes(z)
+    inner, GN = n["ssm_heads"] * n["ssm_dv"], n["groups"] * n["state"]
+    w = w_read = kv = att = 0
+    for mix, ff in nepisun_layers(z, layers):
+        if mix == "mamba2":
+            m = (2 * inner + 2 * GN + n["ssm_heads"]) * H + H * inner
+            kv += B * n["ssm_heads"] * n["state"] * n["ssm_dv"] * 4 * 2
+            att += 4 * T * n["ssm_heads"] * n["state"] * n["ssm_dv"]
+        else:
+            m = 2 * nq * d * H + 2 * nkv * d * H + (nq * d * H if mix == "attention" else 0)
+            reach = (z["window"] + n["keep_first"]) if (mix == "attention_2" and z["window"]) else None
+            kv += B * (min(C, reach) if reach else C) * nkv * 2 * d * 2
+            att += 4 * nq * d * sum(min(p + 1, reach or T) for p in range(T))
+        w += m
+        w_read += m
+        if ff == "dense":
+            w += 3 * I * H
+            w_read += 3 * I * H
+        else:
+            w += 2 * H * (n["top"] * n["expert_ff"] + n["shared_ff"]) + n["experts"] * H
+            w_read += 2 * H * (min(n["experts"], B * n["top"]) * n["expert_ff"] + n["shared_ff"]) + n["experts"] * H
+    return w, kv, att, w_read
+
+
 def bench_designs(args) -> int:
     """Prefill (one prompt of --prefill-tokens in one step) and decode (--batch sequences at --context
     positions, one token a step through captured graphs) of the three designs at equal layer sizes,
@@ -178,6 +243,8 @@ def bench_designs(args) -> int:
         if counts is not None:
             w_elems, kv_bytes, att = counts[0] + V * H, counts[1], counts[2]
             flops = 2 * T * counts[0] + 2 * V * H + att
+            if len(counts) > 3:                               # (what a decode step reads is not what a row multiplies)
+                w_elems = counts[3] + V * H
         return {"prefill_ms": round(pre * 1e3, 3), "prefill_tok_s": round(T / pre),
                 "prefill_frac_of_2.5_pflops": round(flops / pre / 2.5e15, 3),
                 "decode_ms": round(dec * 1e3, 3), "decode_tok_s": round(B / dec),
@@ -190,6 +257,8 @@ def bench_designs(args) -> int:
         row = {}
         if "fanitar" in which:
             row["fanitar"] = measure(fanitar_config(z, L), z, counts=fanitar_counts(z, L, B, C, T))
+        if "nepisun" in which:
+            row["nepisun"] = measure(nepisun_config(z, L), z, counts=nepisun_counts(z, L, B, C, T))
         if "sozetar" in which:
             row["sozetar"] = measure(soz, z)
         if "mistral" in which:
@@ -224,10 +293,10 @@ def main() -> int:
     ap.add_argument("--only", choices=["prefill", "decode", "pipes", "designs"], default=None,
                     help="measure one phase only and print its line to stderr (for profiling); pipes: whether a "
                          "SIMD's matrix and vector pipes overlap (ops.measure_pipes); designs: prefill and decode of "
-                         "the Fanitar and Sozetar designs beside the Mistral design at equal layer sizes (--design-sizes, "
+                         "the Fanitar, Sozetar and Nepisun designs beside the Mistral design at equal layer sizes (--design-sizes, "
                          "--layers, --batch, --context, --prefill-tokens apply)")
     ap.add_argument("--design-names", default="fanitar,sozetar,mistral",
-                    help="with --only designs: which designs to run")
+                    help="with --only designs: which designs to run (of fanitar, sozetar, nepisun, mistral)")
     ap.add_argument("--design-sizes", default="2b,7b,12b",
                     help="with --only designs: which layer sizes to run (of %s)" % ",".join(sorted(DESIGN_SIZES)))
     args = ap.parse_args()

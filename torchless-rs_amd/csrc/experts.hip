@@ -10,6 +10,7 @@
 // The experts run as ONE wide feed-forward: the rows of all up projections stacked (the shared
 // expert's behind them), the activation times the row's weight of the column's expert
 // (`expert_act`), and all down projections side by side: an expert with weight zero adds nothing.
+// Steps of few rows run the chosen experts alone instead (`expert_rows_up`, `expert_rows_down`).
 #include "common.hpp"
 
 namespace tl {
@@ -92,6 +93,100 @@ expert_act_kernel(const float* __restrict__ u, const float* __restrict__ weights
   }
 }
 
+
+// ---- the chosen experts alone, row by row ---------------------------------------------------------------
+// For steps of few rows (fewer chosen experts than there are experts) the wide feed-forward would read every
+// expert's weights to use a few: here a row reads the weights of its own `top` experts and of the shared one,
+// as two products of a matrix with a vector each.  up [E * ff + shared, H] and down [H, E * ff + shared] are
+// the stacked matrices of the wide form, row-major.  Slot k < top of row n is expert chosen[n, k] with the
+// router's weight, slot `top` (with a shared expert) is the shared one with weight 1.
+
+// sum_i a[i] * b[i] over one wave; `vec`: both rows are aligned for loads of 16 bytes and len is a multiple of
+// the vector's length
+template <typename T>
+__device__ __forceinline__ float wave_dot(const T* __restrict__ a, const T* __restrict__ b, int len, bool vec, int lane) {
+  float acc = 0.f;
+  if (vec) {
+    if constexpr (sizeof(T) == 2) {
+      for (int i = lane * 8; i < len; i += WAVE * 8) {
+        const bf16x8 x = *reinterpret_cast<const bf16x8*>(a + i);
+        const bf16x8 y = *reinterpret_cast<const bf16x8*>(b + i);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc = fmaf((float)x[j], (float)y[j], acc);
+      }
+    } else {
+      for (int i = lane * 4; i < len; i += WAVE * 4) {
+        const f32x4 x = *reinterpret_cast<const f32x4*>(a + i);
+        const f32x4 y = *reinterpret_cast<const f32x4*>(b + i);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc = fmaf(x[j], y[j], acc);
+      }
+    }
+  } else {
+    for (int i = lane; i < len; i += WAVE) acc = fmaf(to_f32(a[i]), to_f32(b[i]), acc);
+  }
+  return wave_sum(acc);
+}
+
+constexpr int ER_ROWS = 16;      // outputs of a workgroup: four a wave
+
+// hs[n, k * ff + j] = act(up[e_k * ff + j] . y[n]) * s[n, e_k];  hs[n, top * ff + j] = act(up[E * ff + j] . y[n])
+template <typename T>
+__global__ void __launch_bounds__(256)
+expert_rows_up_kernel(const T* __restrict__ y, int H, const T* __restrict__ up, const int* __restrict__ chosen,
+                      const float* __restrict__ weights, int E, int top, int ff, int shared, int act, bool vec,
+                      T* __restrict__ hs) {
+  const int slots = top + (shared ? 1 : 0);
+  const int n = blockIdx.x / slots, k = blockIdx.x % slots;
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  int base, count;
+  float scale = 1.f;
+  if (k < top) {
+    const int e = chosen[(size_t)n * top + k];
+    base = e * ff;
+    count = ff;
+    scale = weights[(size_t)n * E + e];
+  } else {
+    base = E * ff;
+    count = shared;
+  }
+  const T* row = y + (size_t)n * H;
+  T* out = hs + (size_t)n * (top * ff + shared) + (size_t)k * ff;
+#pragma unroll
+  for (int r = 0; r < ER_ROWS / 4; ++r) {
+    const int j = blockIdx.y * ER_ROWS + wave * (ER_ROWS / 4) + r;
+    if (j >= count) break;
+    float a = fmaxf(wave_dot(up + (size_t)(base + j) * H, row, H, vec, lane), 0.f);
+    if (act == 0) a *= a;
+    if (lane == 0) out[j] = from_f32<T>(a * scale);
+  }
+}
+
+// out[n, c] (+)= sum over the row's slots of down[c, slot's columns] . hs[n, slot's part]
+template <typename T>
+__global__ void __launch_bounds__(256)
+expert_rows_down_kernel(const T* __restrict__ hs, const T* __restrict__ down, const int* __restrict__ chosen, int E, int top,
+                        int ff, int shared, int H, bool vec, int accumulate, float* __restrict__ out) {
+  const int n = blockIdx.x;
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  const int total = E * ff + shared;
+  const T* h = hs + (size_t)n * (top * ff + shared);
+#pragma unroll
+  for (int r = 0; r < ER_ROWS / 4; ++r) {
+    const int c = blockIdx.y * ER_ROWS + wave * (ER_ROWS / 4) + r;
+    if (c >= H) break;
+    const T* w = down + (size_t)c * total;
+    float acc = 0.f;
+    for (int k = 0; k < top; ++k)
+      acc += wave_dot(w + (size_t)chosen[(size_t)n * top + k] * ff, h + (size_t)k * ff, ff, vec, lane);
+    if (shared) acc += wave_dot(w + (size_t)E * ff, h + (size_t)top * ff, shared, vec, lane);
+    if (lane == 0) {
+      float* o = out + (size_t)n * H + c;
+      *o = accumulate ? *o + acc : acc;
+    }
+  }
+}
+
 }  // namespace tl
 
 using namespace tl;
@@ -130,6 +225,48 @@ int tl_expert_act(const float* u, const float* weights, int n, int E, int ff, in
   else
     TL_REQUIRE(false, "expert_act: unknown dtype code %d", dt);
   TL_LAUNCH_CHECK("expert_act");
+  return 0;
+}
+
+// y [n, H], up [E * ff + shared, H], chosen int [n, top], weights [n, E] -> hs [n, top * ff + shared], all of dtype dt
+int tl_expert_rows_up(const void* y, int H, const void* up, const int* chosen, const float* weights, int n, int E, int top, int ff,
+                      int shared, int act, void* hs, int dt, hipStream_t st) {
+  TL_REQUIRE(n >= 0 && H > 0 && E > 0 && top > 0 && top <= E && ff > 0 && shared >= 0 && (act == 0 || act == 1),
+             "expert_rows_up: bad sizes H=%d E=%d top=%d ff=%d shared=%d act=%d", H, E, top, ff, shared, act);
+  TL_REQUIRE(y && up && chosen && weights && hs, "expert_rows_up: a buffer is missing");
+  TL_REQUIRE(dt == DT_F32 || dt == DT_BF16, "expert_rows_up: unknown dtype code %d", dt);
+  if (n == 0) return 0;
+  const int slots = top + (shared ? 1 : 0);
+  const int most = ff > shared ? ff : shared;
+  const dim3 grid(n * slots, (most + ER_ROWS - 1) / ER_ROWS);
+  const int per = dt == DT_BF16 ? 8 : 4;
+  const bool vec = H % per == 0 && (uintptr_t)y % 16 == 0 && (uintptr_t)up % 16 == 0;
+  if (dt == DT_F32)
+    expert_rows_up_kernel<float><<<grid, 256, 0, st>>>((const float*)y, H, (const float*)up, chosen, weights, E, top, ff, shared, act, vec,
+                                                       (float*)hs);
+  else
+    expert_rows_up_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)y, H, (const bf16*)up, chosen, weights, E, top, ff, shared, act, vec,
+                                                      (bf16*)hs);
+  TL_LAUNCH_CHECK("expert_rows_up");
+  return 0;
+}
+
+// hs [n, top * ff + shared], down [H, E * ff + shared] of dtype dt -> out float [n, H], added to or stored
+int tl_expert_rows_down(const void* hs, const void* down, const int* chosen, int n, int E, int top, int ff, int shared, int H,
+                        int accumulate, float* out, int dt, hipStream_t st) {
+  TL_REQUIRE(n >= 0 && H > 0 && E > 0 && top > 0 && top <= E && ff > 0 && shared >= 0, "expert_rows_down: bad sizes H=%d E=%d top=%d ff=%d shared=%d",
+             H, E, top, ff, shared);
+  TL_REQUIRE(hs && down && chosen && out, "expert_rows_down: a buffer is missing");
+  TL_REQUIRE(dt == DT_F32 || dt == DT_BF16, "expert_rows_down: unknown dtype code %d", dt);
+  if (n == 0) return 0;
+  const dim3 grid(n, (H + ER_ROWS - 1) / ER_ROWS);
+  const int per = dt == DT_BF16 ? 8 : 4;
+  const bool vec = ff % per == 0 && shared % per == 0 && (uintptr_t)hs % 16 == 0 && (uintptr_t)down % 16 == 0;
+  if (dt == DT_F32)
+    expert_rows_down_kernel<float><<<grid, 256, 0, st>>>((const float*)hs, (const float*)down, chosen, E, top, ff, shared, H, vec, accumulate, out);
+  else
+    expert_rows_down_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)hs, (const bf16*)down, chosen, E, top, ff, shared, H, vec, accumulate, out);
+  TL_LAUNCH_CHECK("expert_rows_down");
   return 0;
 }
 

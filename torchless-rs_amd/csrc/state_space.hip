@@ -12,7 +12,7 @@
 // and the row's result is rms_parts(y * silu(z)) * w: the gated y cut into equal parts, each
 // divided by its own root mean square (eps inside the root).  dt', a, the state and the sums
 // are float whatever the storage type is; the state lives in a block per sequence,
-// [conv: (taps-1) rows of C channels, the oldest first | S: heads * N * dv], and is carried
+// [conv: (taps-1) rows of C channels, the oldest first | S^T: heads * dv * N], and is carried
 // from step to step.
 #include "common.hpp"
 
@@ -21,7 +21,7 @@ namespace tl {
 constexpr int SSM_MAX_TAPS = 8;
 constexpr int SSM_MAX_N = 256;
 constexpr int SSM_MAX_DV = 256;
-constexpr int SSM_TB = 8;              // rows of a sequence that the recurrence stages at a time
+constexpr int SSM_TB = 16;             // rows of a sequence that the recurrence stages at a time
 
 __device__ __forceinline__ float silu_f(float a) { return a / (1.0f + expf(-a)); }
 __device__ __forceinline__ float softplus_f(float a) { return fmaxf(a, 0.f) + log1pf(expf(-fabsf(a))); }
@@ -78,38 +78,63 @@ ssm_conv_carry_kernel(const float* __restrict__ proj, int width, int off, int C,
   }
 }
 
-// The recurrence, row after row: one workgroup per (head, sequence).  Thread (slice s, column d)
-// keeps rows s, s + nsl, ... of column d of the state in registers (R of them at most).
+// One row a sequence: the convolution and the block's shift in one pass (a thread reads and writes its own
+// channel of its own sequence alone).
+template <typename T>
+__global__ void __launch_bounds__(256)
+ssm_conv_single_kernel(const float* __restrict__ proj, int width, int off, int C, const float* __restrict__ w,
+                       const float* __restrict__ bias, int taps, float* __restrict__ conv_state, long long stride,
+                       const int* __restrict__ slots, T* __restrict__ out) {
+  const int b = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= C) return;
+  float* st = conv_state + (long long)slots[b] * stride;
+  const float cur = proj[(size_t)b * width + off + c];
+  float acc = bias ? bias[c] : 0.f;
+  for (int j = 0; j < taps - 1; ++j) {
+    const float old = st[(size_t)j * C + c];
+    acc = fmaf(w[(size_t)c * taps + j], old, acc);
+    if (j > 0) st[(size_t)(j - 1) * C + c] = old;
+  }
+  acc = fmaf(w[(size_t)c * taps + taps - 1], cur, acc);
+  if (taps > 1) st[(size_t)(taps - 2) * C + c] = cur;
+  out[(size_t)b * C + c] = from_f32<T>(silu_f(acc));
+}
+
+// The recurrence, row after row: one workgroup per (head, sequence, part of the head's columns).  A head's state
+// is kept column by column, S^T [dv, N].  The workgroup takes `dvb` columns; `nsl` neighbouring lanes (a power of
+// two, at most a wave) share a column: lane s keeps rows s, s + nsl, ... of it in registers (R at most) and the
+// column's sum over the rows is a butterfly over those lanes, so a row of the sequence costs no barrier.  The
+// rows' x, B, C, dt' and decay are staged SSM_TB rows at a time.
 template <typename T, int R>
 __global__ void __launch_bounds__(256)
-ssm_scan_kernel(const T* __restrict__ u, int C, int inner, int G, int N, int heads, int dv, const float* __restrict__ proj,
-                int width, int dt_off, const float* __restrict__ dt_bias, const float* __restrict__ A_log,
-                const float* __restrict__ Dw, float* __restrict__ state, long long stride, const int* __restrict__ cu_seqlens,
-                const int* __restrict__ slots, float* __restrict__ y) {
+ssm_scan_kernel(const T* __restrict__ u, int C, int inner, int G, int N, int heads, int dv, int dvb, int nsl,
+                const float* __restrict__ proj, int width, int dt_off, const float* __restrict__ dt_bias,
+                const float* __restrict__ A_log, const float* __restrict__ Dw, float* __restrict__ state, long long stride,
+                const int* __restrict__ cu_seqlens, const int* __restrict__ slots, float* __restrict__ y) {
   __shared__ float xs[SSM_TB][SSM_MAX_DV], Bs[SSM_TB][SSM_MAX_N], Cs[SSM_TB][SSM_MAX_N];
   __shared__ float as[SSM_TB], dts[SSM_TB];
-  __shared__ float part[2][256];
-  const int h = blockIdx.x, b = blockIdx.y;
+  const int h = blockIdx.x, b = blockIdx.y, d0 = blockIdx.z * dvb;
   const int g = h / (heads / G);
   const int t = threadIdx.x;
-  const int nsl = 256 / dv;
-  const bool active = t < nsl * dv;
-  const int d = t % dv, s = t / dv;
+  const int s = t % nsl, dl = t / nsl;
+  const bool active = dl < dvb;
+  const int d = d0 + (active ? dl : 0);
   const int row0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - row0;
-  float* S_g = state + (long long)slots[b] * stride + (size_t)h * N * dv;
+  float* S_g = state + (long long)slots[b] * stride + (size_t)h * N * dv + (size_t)d * N;
   float S[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int nr = s + r * nsl;
-    S[r] = (active && nr < N) ? S_g[(size_t)nr * dv + d] : 0.f;
+    S[r] = (active && nr < N) ? S_g[nr] : 0.f;
   }
   const float neg_rate = -expf(A_log[h]);
   const float bias = dt_bias[h], skip = Dw[h];
-  int parity = 0;
   for (int i0 = 0; i0 < n_new; i0 += SSM_TB) {
     const int tb = min(SSM_TB, n_new - i0);
     __syncthreads();                     // the last batch's rows have been read
-    for (int e = t; e < tb * dv; e += 256) xs[e / dv][e % dv] = to_f32(u[(size_t)(row0 + i0 + e / dv) * C + h * dv + e % dv]);
+    for (int e = t; e < tb * dvb; e += 256)
+      xs[e / dvb][e % dvb] = to_f32(u[(size_t)(row0 + i0 + e / dvb) * C + h * dv + d0 + e % dvb]);
     for (int e = t; e < tb * N; e += 256) {
       const size_t at = (size_t)(row0 + i0 + e / N) * C + inner + g * N + e % N;
       Bs[e / N][e % N] = to_f32(u[at]);
@@ -122,9 +147,9 @@ ssm_scan_kernel(const T* __restrict__ u, int C, int inner, int G, int N, int hea
     }
     __syncthreads();
     for (int i = 0; i < tb; ++i) {
-      const float a = as[i], dt = dts[i];
-      const float x = active ? xs[i][d] : 0.f;
-      const float dtx = dt * x;
+      const float a = as[i];
+      const float x = active ? xs[i][dl] : 0.f;
+      const float dtx = dts[i] * x;
       float acc = 0.f;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
@@ -134,20 +159,14 @@ ssm_scan_kernel(const T* __restrict__ u, int C, int inner, int G, int N, int hea
           acc = fmaf(S[r], Cs[i][nr], acc);
         }
       }
-      part[parity][t] = acc;
-      __syncthreads();
-      if (t < dv) {
-        float sum = 0.f;
-        for (int q = 0; q < nsl; ++q) sum += part[parity][q * dv + t];
-        y[(size_t)(row0 + i0 + i) * inner + h * dv + t] = fmaf(skip, xs[i][t], sum);
-      }
-      parity ^= 1;
+      for (int o = nsl >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, WAVE);
+      if (s == 0 && active) y[(size_t)(row0 + i0 + i) * inner + h * dv + d] = fmaf(skip, x, acc);
     }
   }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int nr = s + r * nsl;
-    if (active && nr < N) S_g[(size_t)nr * dv + d] = S[r];
+    if (active && nr < N) S_g[nr] = S[r];
   }
 }
 
@@ -179,13 +198,14 @@ ssm_gate_norm_kernel(const float* __restrict__ y, const float* __restrict__ proj
 using namespace tl;
 
 template <typename T>
-static int scan_launch(int R, dim3 grid, hipStream_t st, const T* u, int C, int inner, int G, int N, int heads, int dv,
-                       const float* proj, int width, int dt_off, const float* dt_bias, const float* A_log, const float* D,
+static int scan_launch(int R, dim3 grid, hipStream_t st, const T* u, int C, int inner, int G, int N, int heads, int dv, int dvb,
+                       int nsl, const float* proj, int width, int dt_off, const float* dt_bias, const float* A_log, const float* D,
                        float* state, long long stride, const int* cu, const int* slots, float* y) {
-#define TL_SCAN(RR)                                                                                                     \
-  ssm_scan_kernel<T, RR><<<grid, 256, 0, st>>>(u, C, inner, G, N, heads, dv, proj, width, dt_off, dt_bias, A_log, D, state, \
-                                               stride, cu, slots, y)
-  if (R <= 8) TL_SCAN(8);
+#define TL_SCAN(RR)                                                                                                       \
+  ssm_scan_kernel<T, RR><<<grid, 256, 0, st>>>(u, C, inner, G, N, heads, dv, dvb, nsl, proj, width, dt_off, dt_bias, A_log, D, \
+                                               state, stride, cu, slots, y)
+  if (R <= 4) TL_SCAN(4);
+  else if (R <= 8) TL_SCAN(8);
   else if (R <= 16) TL_SCAN(16);
   else if (R <= 32) TL_SCAN(32);
   else TL_SCAN(64);
@@ -193,12 +213,20 @@ static int scan_launch(int R, dim3 grid, hipStream_t st, const T* u, int C, int 
   return 0;
 }
 
+// How a head's dv columns are cut over workgroups and a workgroup's 256 lanes over its columns.
+static void scan_shape(int N, int dv, int& dvb, int& nsl, int& R) {
+  dvb = dv % 16 == 0 ? 16 : dv;
+  nsl = 1;
+  while (nsl * 2 <= WAVE && nsl * 2 * dvb <= 256 && nsl < N) nsl *= 2;
+  R = (N + nsl - 1) / nsl;
+}
+
 extern "C" {
 
 // proj [n, width]: the convolution's input are its columns off .. off + C - 1.
 int tl_ssm_conv(const float* proj, int width, int off, int C, const float* w, const float* bias, int taps,
                 float* conv_state, long long stride, const int* row_seq, const int* cu_seqlens, const int* slots, int n,
-                int B, void* out, int dt, hipStream_t st) {
+                int B, int single, void* out, int dt, hipStream_t st) {
   TL_REQUIRE(n >= 0 && B >= 0 && C > 0 && off >= 0 && off + C <= width, "ssm_conv: bad sizes n=%d C=%d off=%d width=%d", n, C,
              off, width);
   TL_REQUIRE(taps >= 1 && taps <= SSM_MAX_TAPS, "ssm_conv: %d taps (1..%d)", taps, SSM_MAX_TAPS);
@@ -206,6 +234,16 @@ int tl_ssm_conv(const float* proj, int width, int off, int C, const float* w, co
   TL_REQUIRE(stride >= (long long)(taps - 1) * C, "ssm_conv: a sequence's block is too small for %d rows of %d", taps - 1, C);
   TL_REQUIRE(dt == DT_F32 || dt == DT_BF16, "ssm_conv: unknown dtype code %d", dt);
   if (n == 0 || B == 0) return 0;
+  TL_REQUIRE(!single || n == B, "ssm_conv: %d rows of %d sequences are not one row each", n, B);
+  if (single) {        // one row a sequence (row b is sequence b's): the block is shifted in the same pass
+    const dim3 grid1(B, (C + 255) / 256);
+    if (dt == DT_F32)
+      ssm_conv_single_kernel<float><<<grid1, 256, 0, st>>>(proj, width, off, C, w, bias, taps, conv_state, stride, slots, (float*)out);
+    else
+      ssm_conv_single_kernel<bf16><<<grid1, 256, 0, st>>>(proj, width, off, C, w, bias, taps, conv_state, stride, slots, (bf16*)out);
+    TL_LAUNCH_CHECK("ssm_conv_single");
+    return 0;
+  }
   const dim3 grid(n, (C + 255) / 256);
   if (dt == DT_F32)
     ssm_conv_kernel<float><<<grid, 256, 0, st>>>(proj, width, off, C, w, bias, taps, conv_state, stride, row_seq, cu_seqlens,
@@ -233,18 +271,19 @@ int tl_ssm_scan(const void* u, int dt, int C, int G, int N, int heads, int dv, c
   const int inner = heads * dv;
   TL_REQUIRE(C == inner + 2 * G * N && dt_off >= 0 && dt_off + heads <= width, "ssm_scan: %d channels for heads=%d dv=%d G=%d N=%d", C,
              heads, dv, G, N);
-  const int nsl = 256 / dv, R = (N + nsl - 1) / nsl;
+  int dvb, nsl, R;
+  scan_shape(N, dv, dvb, nsl, R);
   TL_REQUIRE(R <= 64, "ssm_scan: a state of %d x %d gives a thread %d rows (at most 64)", N, dv, R);
   TL_REQUIRE(stride >= (long long)heads * N * dv, "ssm_scan: a sequence's block is too small");
   TL_REQUIRE(u && proj && dt_bias && A_log && D && state && cu_seqlens && slots && y, "ssm_scan: a buffer is missing");
   TL_REQUIRE(dt == DT_F32 || dt == DT_BF16, "ssm_scan: unknown dtype code %d", dt);
   if (n == 0 || B == 0) return 0;
-  const dim3 grid(heads, B);
+  const dim3 grid(heads, B, dv / dvb);
   if (dt == DT_F32)
-    scan_launch<float>(R, grid, st, (const float*)u, C, inner, G, N, heads, dv, proj, width, dt_off, dt_bias, A_log, D, state, stride,
+    scan_launch<float>(R, grid, st, (const float*)u, C, inner, G, N, heads, dv, dvb, nsl, proj, width, dt_off, dt_bias, A_log, D, state, stride,
                        cu_seqlens, slots, y);
   else
-    scan_launch<bf16>(R, grid, st, (const bf16*)u, C, inner, G, N, heads, dv, proj, width, dt_off, dt_bias, A_log, D, state, stride,
+    scan_launch<bf16>(R, grid, st, (const bf16*)u, C, inner, G, N, heads, dv, dvb, nsl, proj, width, dt_off, dt_bias, A_log, D, state, stride,
                       cu_seqlens, slots, y);
   TL_LAUNCH_CHECK("ssm_scan");
   return 0;

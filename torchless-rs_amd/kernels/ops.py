@@ -726,11 +726,12 @@ def head_prepare(proj: torch.Tensor, row_pos, rotation, terms: HeadTerms, nq: in
 
 # ---- the state-space mixer ---------------------------------------------------------------------------
 def ssm_conv(proj: torch.Tensor, off: int, C: int, w: torch.Tensor, bias, conv_state: torch.Tensor, row_seq, cu_seqlens,
-             slots, out: torch.Tensor) -> None:
+             slots, out: torch.Tensor, single: bool = False) -> None:
     """The short causal convolution of a state-space mixer over the columns off .. off + C - 1 of proj
     (float32 [n, width]) and silu: out[n, c] = silu(bias[c] + sum_j w[c, j] * u[row - (taps - 1 - j), c]).  Rows
     before the step come from the sequence's block `conv_state` [slots, >= (taps - 1) * C] (float32, the
-    oldest row first, zeros before the start), which afterwards holds the step's last taps - 1 inputs."""
+    oldest row first, zeros before the start), which afterwards holds the step's last taps - 1 inputs.  `single`: every
+    sequence brings one row (row b is sequence b's): one pass does both."""
     n, width = proj.shape
     taps = w.shape[1]
     B = slots.shape[0]
@@ -747,8 +748,8 @@ def ssm_conv(proj: torch.Tensor, off: int, C: int, w: torch.Tensor, bias, conv_s
     if conv_state.shape[1] < (taps - 1) * C:
         raise KernelError(f"ssm_conv: a block of {conv_state.shape[1]} for {taps - 1} rows of {C}")
     _check(lib().tl_ssm_conv(_p(proj), width, int(off), int(C), _p(w), _p(bias), taps, _p(conv_state),
-                             ctypes.c_longlong(conv_state.stride(0)), _p(row_seq), _p(cu_seqlens), _p(slots), n, B, _p(out),
-                             _code(out.dtype), _stream()))
+                             ctypes.c_longlong(conv_state.stride(0)), _p(row_seq), _p(cu_seqlens), _p(slots), n, B, int(bool(single)),
+                             _p(out), _code(out.dtype), _stream()))
 
 
 def ssm_scan(u: torch.Tensor, proj: torch.Tensor, dt_off: int, G: int, N: int, heads: int, dv: int, dt_bias, A_log, D,
@@ -821,6 +822,38 @@ def expert_act(u: torch.Tensor, weights: Optional[torch.Tensor], E: int, ff: int
     _req(out, "expert_act.out", None, (n, total))
     _check(lib().tl_expert_act(_p(u), _p(weights) if E else None, n, int(E), int(ff), total, EXPERT_ACTIVATIONS[activation],
                                _p(out), _code(out.dtype), _stream()))
+
+
+def expert_rows_up(y: torch.Tensor, up: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor, ff: int, shared: int,
+                   activation: str, hs: torch.Tensor) -> None:
+    """The chosen experts' first halves, row by row: hs[n, k*ff + j] = act(up[chosen[n,k]*ff + j] . y[n]) * weights[n, chosen[n,k]]
+    and, behind them, the shared expert's `shared` rows with weight 1.  up [E*ff + shared, H] and y [n, H] of one dtype."""
+    n, H = y.shape
+    top, E = chosen.shape[1], weights.shape[1]
+    if activation not in EXPERT_ACTIVATIONS:
+        raise KernelError(f"expert_rows_up: no function {activation!r}; there are {sorted(EXPERT_ACTIVATIONS)}")
+    _req(y, "expert_rows_up.y")
+    _req(up, "expert_rows_up.up", y.dtype, (E * ff + shared, H))
+    _req(chosen, "expert_rows_up.chosen", torch.int32, (n, top))
+    _req(weights, "expert_rows_up.weights", torch.float32, (n, E))
+    _req(hs, "expert_rows_up.hs", y.dtype, (n, top * ff + shared))
+    _check(lib().tl_expert_rows_up(_p(y), H, _p(up), _p(chosen), _p(weights), n, E, top, int(ff), int(shared),
+                                   EXPERT_ACTIVATIONS[activation], _p(hs), _code(y.dtype), _stream()))
+
+
+def expert_rows_down(hs: torch.Tensor, down: torch.Tensor, chosen: torch.Tensor, E: int, ff: int, shared: int, out: torch.Tensor,
+                     accumulate: bool = False) -> None:
+    """out[n] (+)= sum over the row's chosen experts (and the shared one) of their down projections of their part of
+    hs [n, top*ff + shared]; down [H, E*ff + shared] of hs's dtype, out float32 [n, H]."""
+    n = hs.shape[0]
+    top = chosen.shape[1]
+    H = down.shape[0]
+    _req(hs, "expert_rows_down.hs", None, (n, top * ff + shared))
+    _req(down, "expert_rows_down.down", hs.dtype, (H, E * ff + shared))
+    _req(chosen, "expert_rows_down.chosen", torch.int32, (n, top))
+    _req(out, "expert_rows_down.out", torch.float32, (n, H))
+    _check(lib().tl_expert_rows_down(_p(hs), _p(down), _p(chosen), n, int(E), top, int(ff), int(shared), H, int(bool(accumulate)),
+                                     _p(out), _code(hs.dtype), _stream()))
 
 
 def take_tokens(src: torch.Tensor, idx: torch.Tensor, vocab: int, tokens: torch.Tensor) -> None:

@@ -14,8 +14,14 @@ All experts run as ONE wide feed-forward: their up projections stacked by rows (
 expert's behind them), the activation times the row's weight of the column's expert, which is
 zero for an expert that was not chosen, and their down projections side by side.  That is two
 products of the framework's own kinds and no gather or scatter, whatever the tokens choose; it
-reads every expert's weights in every step, as a step of several sequences does anyway, and
-multiplies `n_experts / top` times what the chosen experts alone would.
+reads every expert's weights in every step, as a step of many rows does anyway, and multiplies
+`n_experts / top` times what the chosen experts alone would.
+
+A step of few rows (rows * top <= n_experts: the rows cannot use every expert) runs the chosen
+experts alone: per row two products of its experts' matrices with a vector
+(`ops.expert_rows_up`, `ops.expert_rows_down`), which read `top` experts' weights a row and
+nothing else.  Both ways round the hidden activations, times the router's weight, to the
+compute dtype and sum in float32.
 """
 from __future__ import annotations
 
@@ -25,7 +31,7 @@ import torch
 
 from ..kernels import ops
 from ..weights.binding import WeightSpec
-from .base import FeedForward, register_part
+from .base import FeedForward, flush_pending, register_part
 from .linear import Linear
 
 
@@ -124,6 +130,20 @@ class RoutedExperts(FeedForward):
         self.down = Linear(torch.cat(downs, dim=1), tiled=True)      # [H, E * ff + shared]
         self.router = tensors[p + nm["router"]].to(torch.float32).contiguous()
 
+    def few_rows(self, y: torch.Tensor) -> bool:
+        """Do the rows of `y` run their chosen experts alone?"""
+        return y.shape[0] * self.top <= self.E and self.up.weight.dtype == self.down.weight.dtype == y.dtype
+
+    def _rows(self, ctx, y: torch.Tensor, out: torch.Tensor, accumulate: bool) -> None:
+        n = y.shape[0]
+        ws = ctx.workspace
+        weights = ws.get("experts_w", (n, self.E), torch.float32)
+        chosen = ws.get("experts_chosen", (n, self.top), torch.int32)
+        ops.route(y, self.router, self.groups, self.keep, self.top, weights, chosen)
+        hs = ws.get("experts_hs", (n, self.top * self.ff + self.shared), y.dtype)
+        ops.expert_rows_up(y, self.up.weight, chosen, weights, self.ff, self.shared, self.activation, hs)
+        ops.expert_rows_down(hs, self.down.weight, chosen, self.E, self.ff, self.shared, out, accumulate)
+
     def _hidden(self, ctx, y: torch.Tensor) -> torch.Tensor:
         n = y.shape[0]
         ws = ctx.workspace
@@ -136,9 +156,16 @@ class RoutedExperts(FeedForward):
         return h
 
     def forward(self, ctx, y: torch.Tensor, x: torch.Tensor) -> None:
+        if self.few_rows(y):
+            flush_pending(ctx, x)
+            self._rows(ctx, y, x, True)
+            return
         self.down.add_into(self._hidden(ctx, y), x, ctx, "experts_down_parts")
 
     def produce(self, ctx, y: torch.Tensor, out: torch.Tensor) -> None:
+        if self.few_rows(y):
+            self._rows(ctx, y, out, False)
+            return
         self.down(self._hidden(ctx, y), out)
 
 

@@ -93,7 +93,8 @@ class StateSpaceMixer(Mixer):
         proj = ws.get("ssm_proj", (n, self.width), torch.float32)
         self.proj(y, proj)
         u = ws.get("ssm_u", (n, self.C), ctx.dtype)
-        ops.ssm_conv(proj, self.inner, self.C, self.conv_w, self.conv_b, block, ctx.row_seq, ctx.cu_seqlens, ctx.slots, u)
+        ops.ssm_conv(proj, self.inner, self.C, self.conv_w, self.conv_b, block, ctx.row_seq, ctx.cu_seqlens, ctx.slots, u,
+                     single=ctx.all_single)
         yy = ws.get("ssm_y", (n, self.inner), torch.float32)
         ops.ssm_scan(u, proj, self.inner + self.C, self.G, self.N, self.heads, self.dv, self.dt_bias, self.A_log, self.D,
                      block[:, self.conv_elems:], ctx.cu_seqlens, ctx.slots, yy)
