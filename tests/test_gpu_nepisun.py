@@ -40,12 +40,12 @@ CORES = {"architecture": "Nepisun", "vocab": 256, "width": 128, "norm": {"eps": 
 ]}
 # what a model may happen to make 1 or equal: one head, one group, one expert of which one is used, one group of
 # experts, every group kept, top = experts, a window of one (a position sees itself and the kept ones), no tokens
-# kept, one tap (no convolution), no rotation, values as wide as keys, a single layer that mixes values
+# kept, no window at all, one tap (no convolution), no rotation, values as wide as keys, a single layer that mixes values
 ONES = {"architecture": "Nepisun", "vocab": 96, "width": 32, "norm": {"eps": 1e-4}, "layers": [
     layer(ssm(1, 16, 8, 1, 1, 1), moe(1, 1, 16)),
     layer(attn2(1, 1, 16, 16, 0.25, window=1, keep_first=2), moe(4, 4, 8, groups=(1, 1))),
     layer(attn(2, 2, 8, 8, 0.35, v_mix=True), moe(6, 2, 8, groups=(3, 3), shared=8)),
-    layer(attn2(2, 1, 16, 8, 0.3, rot=(50.0, 16), window=64), dense(16)),
+    layer(attn2(2, 1, 16, 8, 0.3, rot=(50.0, 16)), dense(16)),
     layer(ssm(2, 8, 4, 2, 2, 2), None),
 ]}
 # sizes that no kernel's fast way takes: a width that is no multiple of 8, heads of 12 and 20, three heads, an odd
@@ -171,7 +171,8 @@ def plain_conv_scan(m, w, proj):
 
 SSM_SHAPES = [dict(heads=4, vdim=16, state=24, groups=2, conv=4, norm_groups=2), dict(heads=1, vdim=8, state=4, groups=1, conv=1, norm_groups=1),
               dict(heads=3, vdim=20, state=33, groups=3, conv=7, norm_groups=3), dict(heads=2, vdim=64, state=128, groups=1, conv=2, norm_groups=1),
-              dict(heads=6, vdim=12, state=5, groups=2, conv=3, norm_groups=1), dict(heads=2, vdim=128, state=64, groups=2, conv=4, norm_groups=4)]
+              dict(heads=6, vdim=12, state=5, groups=2, conv=3, norm_groups=1), dict(heads=2, vdim=128, state=64, groups=2, conv=4, norm_groups=4),
+              dict(heads=2, vdim=37, state=70, groups=1, conv=2, norm_groups=2), dict(heads=1, vdim=72, state=256, groups=1, conv=4, norm_groups=3)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

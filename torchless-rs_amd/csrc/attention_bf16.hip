@@ -43,6 +43,20 @@ struct MoreTerms {
   const float* slopes;
   const float* sinks;
   const float* gate;
+  int keep_first;          // with a window: positions 0 .. keep_first - 1 stay visible beside it (the cache then keeps
+                           // every position: no ring of pages)
+};
+
+// The pages that a query at p reads, numbered 0 .. n - 1 in the order they are read: the pages of the window
+// [lo, p], and ahead of them those of the kept first positions that lie before the window's first page.
+struct PageSpan {
+  int pg_lo, kept, n;
+  __device__ __forceinline__ PageSpan(int lo, int p, int keep_first) {
+    pg_lo = lo / PAGE;
+    kept = min((keep_first + PAGE - 1) / PAGE, pg_lo);
+    n = p / PAGE - pg_lo + 1 + kept;
+  }
+  __device__ __forceinline__ int page(int v) const { return v < kept ? v : pg_lo + (v - kept); }
 };
 
 // ------------------------------------------------------------------ prefill --
@@ -184,8 +198,17 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
     jt_first = max(jt_first, cut_lo);
     jt_last = min(jt_last, cut_hi - 1);
   }
-  int f_ring = jt_first % ring_pages;
-  int page_nxt = ((jt_first + 1) * PF_BN <= cached) ? table[(size_t)b * table_stride + f_ring] : 0;
+  // With kept first positions the tiles that hold them, as far as they lie before the window's first tile, go
+  // ahead of the window's (there is no ring of pages then: a tile's page is at its own place in the table).
+  const int keep = (TERMS && window > 0) ? terms.keep_first : 0;
+  const int kept_tiles = (ways == 0) ? min((keep + PF_BN - 1) / PF_BN, jt_first) : 0;
+  const int jt_start = kept_tiles > 0 ? 0 : jt_first;
+  int f_ring = jt_start % ring_pages;
+  int page_nxt = ((jt_start + 1) * PF_BN <= cached) ? table[(size_t)b * table_stride + f_ring] : 0;
+  auto seek = [&](int jt) {
+    f_ring = jt % ring_pages;
+    page_nxt = ((jt + 1) * PF_BN <= cached) ? table[(size_t)b * table_stride + f_ring] : 0;
+  };
   auto fetch = [&](int j0) {
     const int page = page_nxt;
     f_ring = (f_ring + 1 == ring_pages) ? 0 : f_ring + 1;
@@ -280,15 +303,19 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
     }
   };
 
-  if (jt_first <= jt_last) fetch(jt_first * PF_BN);
-  for (int jt = jt_first; jt <= jt_last; ++jt) {
+  if (jt_start <= jt_last) fetch(jt_start * PF_BN);
+  for (int jt = jt_start, nxt; jt <= jt_last; jt = nxt) {
+    nxt = (jt + 1 == kept_tiles) ? jt_first : jt + 1;
     const int j0 = jt * PF_BN;
     __syncthreads();                  // the previous tile has been worked on
     stash();
     __syncthreads();
-    if (jt < jt_last) fetch((jt + 1) * PF_BN);
+    if (nxt <= jt_last) {
+      if (nxt != jt + 1) seek(nxt);
+      fetch(nxt * PF_BN);
+    }
     // does any query of this wave see any key of this tile?
-    if (pw_lo > p_hi || j0 > pw_hi || (window > 0 && j0 + PF_BN - 1 <= pw_lo - window)) continue;
+    if (pw_lo > p_hi || j0 > pw_hi || (window > 0 && j0 + PF_BN - 1 <= pw_lo - window && j0 >= keep)) continue;
 
     f32x16 s[2];
 #pragma unroll
@@ -323,7 +350,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int j = j0 + nb * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-          const bool ok = q_ok && j <= p_me && (window == 0 || j > p_me - window);
+          const bool ok = q_ok && j <= p_me && (window == 0 || j > p_me - window || j < keep);
           s[nb][r] = ok ? s[nb][r] : -INFINITY;
         }
     }
@@ -502,11 +529,12 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
   const int h = kvh * g + min(hl, g - 1);
   const int p = row_pos[b];
   const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
-  const int pg_lo = lo / PAGE, pg_hi = p / PAGE, n_pg = pg_hi - pg_lo + 1;
-  // [my_lo, my_hi): the pages in shares that differ by one at most (65 pages in 8 splits are 8 or 9 each,
-  // not seven times 9 and once 2: the compute units then end together)
-  const int my_lo = pg_lo + (int)((long long)split * n_pg / n_splits);
-  const int my_hi = pg_lo + (int)((long long)(split + 1) * n_pg / n_splits);
+  const int keep = (TERMS && window > 0) ? terms.keep_first : 0;
+  const PageSpan span(lo, p, keep);
+  // [my_lo, my_hi): the pages (as the span numbers them) in shares that differ by one at most (65 pages in 8
+  // splits are 8 or 9 each, not seven times 9 and once 2: the compute units then end together)
+  const int my_lo = (int)((long long)split * span.n / n_splits);
+  const int my_hi = (int)((long long)(split + 1) * span.n / n_splits);
   const size_t head_elems = (size_t)PAGE * d, page_elems = 2 * (size_t)nkv * head_elems;
 
   bf16x8 qreg[KB];
@@ -531,20 +559,24 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
   static_assert(DC_WAVES == 4, "a wave's groups are two pages apart");
   const int* trow = table + (size_t)b * table_stride;
   const int gi0 = 2 * my_lo + wave;
-  int ring = (gi0 / 2) % ring_pages;
+  int ring = span.page(gi0 / 2) % ring_pages;
   int page_nxt = gi0 < 2 * my_hi ? trow[ring] : 0;
   for (int gi = gi0; gi < 2 * my_hi; gi += DC_WAVES) {
-    const int pg = gi / 2, grp = gi % 2;
+    const int pg = span.page(gi / 2), grp = gi % 2;
     const int page = page_nxt;
-    ring += 2;
-    if (ring >= ring_pages) ring -= ring_pages;
-    if (ring >= ring_pages) ring -= ring_pages;          // (a ring of one page)
+    if (span.kept > 0) {
+      ring = span.page((gi + DC_WAVES) / 2);             // (kept positions: no ring, a page's place is its number)
+    } else {
+      ring += 2;
+      if (ring >= ring_pages) ring -= ring_pages;
+      if (ring >= ring_pages) ring -= ring_pages;        // (a ring of one page)
+    }
     if (gi + DC_WAVES < 2 * my_hi) page_nxt = trow[ring];
     const bf16* kbase = pages + (size_t)page * page_elems + (size_t)kvh * head_elems;
     const bf16* vbase = kbase + (size_t)nkv * head_elems;
     {
       const int j0 = pg * PAGE + grp * 32;
-      if (j0 > p || j0 + 31 < lo) continue;
+      if (j0 > p || (j0 + 31 < lo && j0 >= keep)) continue;
       // block bs holds keys j0 + 8 (i/4) + 4 bs + i%4 in its rows i: then a lane's 8 scores of
       // the two blocks are 8 consecutive keys, j0 + 8 kg .. + 7
       // all loads of the group first: keys (two blocks) and values
@@ -590,7 +622,7 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int j = j0 + 8 * kg + e;
-        const bool ok = j <= p && j >= lo;
+        const bool ok = j <= p && (j >= lo || j < keep);
         if constexpr (TERMS) sv[e] = ok ? s[e / 4][e % 4] * scale - slope * (float)(p - j) : -INFINITY;
         else sv[e] = ok ? s[e / 4][e % 4] * scale : -INFINITY;
         tmax = fmaxf(tmax, sv[e]);
@@ -760,9 +792,10 @@ attn_decode_ring_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pag
   const int h = kvh * g + min(hl, g - 1);
   const int p = row_pos[b];
   const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
-  const int pg_lo = lo / PAGE, pg_hi = p / PAGE, n_pg = pg_hi - pg_lo + 1;
-  const int my_lo = pg_lo + (int)((long long)split * n_pg / n_splits);
-  const int my_hi = pg_lo + (int)((long long)(split + 1) * n_pg / n_splits);
+  const int keep = (TERMS && window > 0) ? terms.keep_first : 0;
+  const PageSpan span(lo, p, keep);
+  const int my_lo = (int)((long long)split * span.n / n_splits);
+  const int my_hi = (int)((long long)(split + 1) * span.n / n_splits);
   const int n_st = my_hi - my_lo;                     // this split's pages: the stages
   const size_t head_elems = (size_t)PAGE * D, page_elems = 2 * (size_t)nkv * head_elems;
   auto kkey = [](int r) { return K_CPR >= 16 ? r % 16 : (r / 2) % 8; };   // swizzle of a key's row
@@ -792,7 +825,7 @@ attn_decode_ring_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pag
   int* ids = reinterpret_cast<int*>(dr_smem + NS * STAGE);
   {
     const int* trow = table + (size_t)b * table_stride;
-    for (int st = threadIdx.x; st < n_st; st += DC_WAVES * 64) ids[st] = trow[(my_lo + st) % ring_pages];
+    for (int st = threadIdx.x; st < n_st; st += DC_WAVES * 64) ids[st] = trow[span.page(my_lo + st) % ring_pages];
   }
   __syncthreads();
   auto issue = [&](int st) {
@@ -823,8 +856,8 @@ attn_decode_ring_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pag
     else wait_page_loads_but<0>();
     __builtin_amdgcn_s_barrier();                     // the page is there for all; everyone has left the one before
     if (st + NS - 1 < n_st) issue(st + NS - 1);
-    const int j0 = (my_lo + st) * PAGE + 16 * wave;   // this wave's 16 keys
-    if (j0 > p || j0 + 15 < lo) continue;             // none of them visible
+    const int j0 = span.page(my_lo + st) * PAGE + 16 * wave;   // this wave's 16 keys
+    if (j0 > p || (j0 + 15 < lo && j0 >= keep)) continue;      // none of them visible
     const unsigned char* slot = dr_smem + (st % NS) * STAGE;
     bf16x8 kreg[KB];
 #pragma unroll
@@ -844,8 +877,9 @@ attn_decode_ring_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pag
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int j = j0 + 4 * kg + r;
-      if constexpr (TERMS) sv[r] = (j <= p && j >= lo) ? s[r] * scale - slope * (float)(p - j) : -INFINITY;
-      else sv[r] = (j <= p && j >= lo) ? s[r] * scale : -INFINITY;
+      const bool ok = j <= p && (j >= lo || j < keep);
+      if constexpr (TERMS) sv[r] = ok ? s[r] * scale - slope * (float)(p - j) : -INFINITY;
+      else sv[r] = ok ? s[r] * scale : -INFINITY;
       tmax = fmaxf(tmax, sv[r]);
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
@@ -1241,9 +1275,11 @@ extern "C" int tl_attn_prefill_terms_bf16(const void* q, const void* k_new, cons
                                           const int* tile_off, const void* pages, const int* table, int table_stride,
                                           int ring_pages, const int* row_pos, const int* cu_seqlens,
                                           const int* n_cached, int B, int n_tiles, int nq, int nkv, int d,
-                                          int window, float scale, const float* slopes, const float* sinks,
-                                          const float* gate, void* out, hipStream_t st) {
-  const MoreTerms terms{slopes, sinks, gate};
+                                          int window, int keep_first, float scale, const float* slopes,
+                                          const float* sinks, const float* gate, void* out, hipStream_t st) {
+  TL_REQUIRE(keep_first >= 0 && (keep_first == 0 || window == 0 || (long long)ring_pages * PAGE >= (1LL << 24)),
+             "attn_prefill: first positions that stay visible beside a window need a cache that keeps every position");
+  const MoreTerms terms{slopes, sinks, gate, window > 0 ? keep_first : 0};
   return attn_prefill_entry(q, k_new, vt_new, vt_cols, tile_off, pages, table, table_stride, ring_pages, row_pos,
                             cu_seqlens, n_cached, B, n_tiles, nq, nkv, d, window, scale, out, nullptr, nullptr, 0,
                             nullptr, 0, 0, 0, st, &terms);
@@ -1285,9 +1321,12 @@ extern "C" int tl_attn_decode_bf16(const void* q, const void* pages, const int* 
 // The same with more terms on the scores (slopes [nq], sinks [nq], gate [B, nq]; each may be null)
 extern "C" int tl_attn_decode_terms_bf16(const void* q, const void* pages, const int* table, int table_stride,
                                          int ring_pages, const int* row_pos, int B, int nq, int nkv, int d,
-                                         int window, float scale, int n_splits, float* part, const float* slopes,
-                                         const float* sinks, const float* gate, void* out, hipStream_t st) {
-  const MoreTerms terms{slopes, sinks, gate};
+                                         int window, int keep_first, float scale, int n_splits, float* part,
+                                         const float* slopes, const float* sinks, const float* gate, void* out,
+                                         hipStream_t st) {
+  TL_REQUIRE(keep_first >= 0 && (keep_first == 0 || window == 0 || (long long)ring_pages * PAGE >= (1LL << 24)),
+             "attn_decode: first positions that stay visible beside a window need a cache that keeps every position");
+  const MoreTerms terms{slopes, sinks, gate, window > 0 ? keep_first : 0};
   return attn_decode_entry(q, pages, table, table_stride, ring_pages, row_pos, B, nq, nkv, d, window, scale, n_splits,
                            part, out, st, &terms);
 }

@@ -30,9 +30,16 @@ route_kernel(const T* __restrict__ h, int W, const float* __restrict__ wr, int E
   const T* row = h + (size_t)n * W;
   for (int e = wave; e < E; e += 4) {
     const float* w = wr + (size_t)e * W;
-    float dot = 0.f;
-    for (int c = lane; c < W; c += WAVE) dot = fmaf(w[c], to_f32(row[c]), dot);
-    dot = wave_sum(dot);
+    float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;      // four chains: the loads of one do not wait for another's sum
+    int c = lane;
+    for (; c + 3 * WAVE < W; c += 4 * WAVE) {
+      d0 = fmaf(w[c], to_f32(row[c]), d0);
+      d1 = fmaf(w[c + WAVE], to_f32(row[c + WAVE]), d1);
+      d2 = fmaf(w[c + 2 * WAVE], to_f32(row[c + 2 * WAVE]), d2);
+      d3 = fmaf(w[c + 3 * WAVE], to_f32(row[c + 3 * WAVE]), d3);
+    }
+    for (; c < W; c += WAVE) d0 = fmaf(w[c], to_f32(row[c]), d0);
+    float dot = wave_sum((d0 + d1) + (d2 + d3));
     if (lane == 0) s_s[e] = dot;
   }
   __syncthreads();

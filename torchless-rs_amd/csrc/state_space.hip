@@ -112,8 +112,12 @@ ssm_scan_kernel(const T* __restrict__ u, int C, int inner, int G, int N, int hea
                 const float* __restrict__ proj, int width, int dt_off, const float* __restrict__ dt_bias,
                 const float* __restrict__ A_log, const float* __restrict__ Dw, float* __restrict__ state, long long stride,
                 const int* __restrict__ cu_seqlens, const int* __restrict__ slots, float* __restrict__ y) {
-  __shared__ float xs[SSM_TB][SSM_MAX_DV], Bs[SSM_TB][SSM_MAX_N], Cs[SSM_TB][SSM_MAX_N];
-  __shared__ float as[SSM_TB], dts[SSM_TB];
+  extern __shared__ float ssm_lds[];
+  float* xs = ssm_lds;                 // [SSM_TB][dvb]
+  float* Bs = xs + SSM_TB * dvb;       // [SSM_TB][N]
+  float* Cs = Bs + SSM_TB * N;         // [SSM_TB][N]
+  float* as = Cs + SSM_TB * N;         // [SSM_TB]
+  float* dts = as + SSM_TB;            // [SSM_TB]
   const int h = blockIdx.x, b = blockIdx.y, d0 = blockIdx.z * dvb;
   const int g = h / (heads / G);
   const int t = threadIdx.x;
@@ -134,11 +138,11 @@ ssm_scan_kernel(const T* __restrict__ u, int C, int inner, int G, int N, int hea
     const int tb = min(SSM_TB, n_new - i0);
     __syncthreads();                     // the last batch's rows have been read
     for (int e = t; e < tb * dvb; e += 256)
-      xs[e / dvb][e % dvb] = to_f32(u[(size_t)(row0 + i0 + e / dvb) * C + h * dv + d0 + e % dvb]);
+      xs[e] = to_f32(u[(size_t)(row0 + i0 + e / dvb) * C + h * dv + d0 + e % dvb]);
     for (int e = t; e < tb * N; e += 256) {
       const size_t at = (size_t)(row0 + i0 + e / N) * C + inner + g * N + e % N;
-      Bs[e / N][e % N] = to_f32(u[at]);
-      Cs[e / N][e % N] = to_f32(u[at + (size_t)G * N]);
+      Bs[e] = to_f32(u[at]);
+      Cs[e] = to_f32(u[at + (size_t)G * N]);
     }
     if (t < tb) {
       const float dt = softplus_f(proj[(size_t)(row0 + i0 + t) * width + dt_off + h] + bias);
@@ -146,22 +150,35 @@ ssm_scan_kernel(const T* __restrict__ u, int C, int inner, int G, int N, int hea
       as[t] = expf(neg_rate * dt);
     }
     __syncthreads();
-    for (int i = 0; i < tb; ++i) {
-      const float a = as[i];
-      const float x = active ? xs[i][dl] : 0.f;
-      const float dtx = dts[i] * x;
-      float acc = 0.f;
+    // the batch's rows one after the other, each lane its own rows of the state; the sums over a column's lanes
+    // wait until the batch is through, so that no row waits for a butterfly
+    float sums[SSM_TB];
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        const int nr = s + r * nsl;
-        if (nr < N) {
-          S[r] = fmaf(a, S[r], Bs[i][nr] * dtx);
-          acc = fmaf(S[r], Cs[i][nr], acc);
+    for (int i = 0; i < SSM_TB; ++i) {
+      sums[i] = 0.f;
+      if (i < tb) {
+        const float a = as[i];
+        const float dtx = dts[i] * (active ? xs[i * dvb + dl] : 0.f);
+        float acc = 0.f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const int nr = s + r * nsl;
+          if (nr < N) {
+            S[r] = fmaf(a, S[r], Bs[i * N + nr] * dtx);
+            acc = fmaf(S[r], Cs[i * N + nr], acc);
+          }
         }
+        sums[i] = acc;
       }
-      for (int o = nsl >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, WAVE);
-      if (s == 0 && active) y[(size_t)(row0 + i0 + i) * inner + h * dv + d] = fmaf(skip, x, acc);
     }
+    for (int o = nsl >> 1; o > 0; o >>= 1) {
+#pragma unroll
+      for (int i = 0; i < SSM_TB; ++i) sums[i] += __shfl_xor(sums[i], o, WAVE);
+    }
+#pragma unroll
+    for (int i = 0; i < SSM_TB; ++i)          // every lane of a column holds the sums: lane s writes rows s, s + nsl, ...
+      if (i < tb && (i & (nsl - 1)) == s && active)
+        y[(size_t)(row0 + i0 + i) * inner + h * dv + d] = fmaf(skip, xs[i * dvb + dl], sums[i]);
   }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
@@ -198,11 +215,11 @@ ssm_gate_norm_kernel(const float* __restrict__ y, const float* __restrict__ proj
 using namespace tl;
 
 template <typename T>
-static int scan_launch(int R, dim3 grid, hipStream_t st, const T* u, int C, int inner, int G, int N, int heads, int dv, int dvb,
+static int scan_launch(int R, dim3 grid, size_t lds, hipStream_t st, const T* u, int C, int inner, int G, int N, int heads, int dv, int dvb,
                        int nsl, const float* proj, int width, int dt_off, const float* dt_bias, const float* A_log, const float* D,
                        float* state, long long stride, const int* cu, const int* slots, float* y) {
 #define TL_SCAN(RR)                                                                                                       \
-  ssm_scan_kernel<T, RR><<<grid, 256, 0, st>>>(u, C, inner, G, N, heads, dv, dvb, nsl, proj, width, dt_off, dt_bias, A_log, D, \
+  ssm_scan_kernel<T, RR><<<grid, 256, lds, st>>>(u, C, inner, G, N, heads, dv, dvb, nsl, proj, width, dt_off, dt_bias, A_log, D, \
                                                state, stride, cu, slots, y)
   if (R <= 4) TL_SCAN(4);
   else if (R <= 8) TL_SCAN(8);
@@ -215,7 +232,12 @@ static int scan_launch(int R, dim3 grid, hipStream_t st, const T* u, int C, int 
 
 // How a head's dv columns are cut over workgroups and a workgroup's 256 lanes over its columns.
 static void scan_shape(int N, int dv, int& dvb, int& nsl, int& R) {
-  dvb = dv % 16 == 0 ? 16 : dv;
+  dvb = dv;                                   // the largest part of dv of at most 16 columns, if it has one of 4 or more
+  for (int c = 16; c >= 4; --c)
+    if (dv % c == 0) {
+      dvb = c;
+      break;
+    }
   nsl = 1;
   while (nsl * 2 <= WAVE && nsl * 2 * dvb <= 256 && nsl < N) nsl *= 2;
   R = (N + nsl - 1) / nsl;
@@ -279,11 +301,12 @@ int tl_ssm_scan(const void* u, int dt, int C, int G, int N, int heads, int dv, c
   TL_REQUIRE(dt == DT_F32 || dt == DT_BF16, "ssm_scan: unknown dtype code %d", dt);
   if (n == 0 || B == 0) return 0;
   const dim3 grid(heads, B, dv / dvb);
+  const size_t lds = sizeof(float) * ((size_t)SSM_TB * (dvb + 2 * N) + 2 * SSM_TB);
   if (dt == DT_F32)
-    scan_launch<float>(R, grid, st, (const float*)u, C, inner, G, N, heads, dv, dvb, nsl, proj, width, dt_off, dt_bias, A_log, D, state, stride,
+    scan_launch<float>(R, grid, lds, st, (const float*)u, C, inner, G, N, heads, dv, dvb, nsl, proj, width, dt_off, dt_bias, A_log, D, state, stride,
                        cu_seqlens, slots, y);
   else
-    scan_launch<bf16>(R, grid, st, (const bf16*)u, C, inner, G, N, heads, dv, dvb, nsl, proj, width, dt_off, dt_bias, A_log, D, state, stride,
+    scan_launch<bf16>(R, grid, lds, st, (const bf16*)u, C, inner, G, N, heads, dv, dvb, nsl, proj, width, dt_off, dt_bias, A_log, D, state, stride,
                       cu_seqlens, slots, y);
   TL_LAUNCH_CHECK("ssm_scan");
   return 0;

@@ -462,11 +462,6 @@ def scored_on_matrix_cores(dtype: torch.dtype, dk: int, dv: int) -> bool:
     return dtype == torch.bfloat16 and dk == dv and dk % 16 == 0 and 16 <= dk <= 256
 
 
-def terms_on_matrix_cores(terms: ScoreTerms) -> bool:
-    """Do the matrix-core kernels know every term of `terms`?"""
-    return not terms.keep_first
-
-
 def _terms_args(terms: ScoreTerms, gate, n: int, nq: int):
     if terms.slopes is not None:
         _req(terms.slopes, "attn_scored.slopes", torch.float32, (nq,))
@@ -485,15 +480,19 @@ def attention_scored(q, k_new, v_new, pages, nkv: int, dv: int, table, ring_page
     in the TERMS variant of the kernels of `attention` (the latter takes the step's values
     transposed, `vt_new`); everything else in the plain kernel."""
     n, nq, dk = q.shape
-    fast = scored_on_matrix_cores(q.dtype, dk, dv) and pages.dim() == 5 and terms_on_matrix_cores(terms)
+    fast = scored_on_matrix_cores(q.dtype, dk, dv) and pages.dim() == 5
     if fast and k_new is None and ctx.all_single:
-        splits = decode_splits(n, nq, nkv, table.shape[1], compute_units(q.device), dk)
+        most_pages = table.shape[1]
+        if terms.window:          # (kept first positions: the table holds every page, a row reads the window's and the kept ones)
+            most_pages = min(most_pages, -(-terms.window // PAGE) + 1 + -(-int(terms.keep_first or 0) // PAGE))
+        splits = decode_splits(n, nq, nkv, most_pages, compute_units(q.device), dk)
         part = ctx.workspace.get("attn_part", (n * nq * splits * (dk + 2),), torch.float32)
         _decode_args(q, pages, table, ctx.row_pos, part, out, splits)
         slopes, sinks, gt = _terms_args(terms, gate, n, nq)
         _check(lib().tl_attn_decode_terms_bf16(_p(q), _p(pages), _p(table), table.shape[1], ring_pages, _p(ctx.row_pos),
-                                               n, nq, nkv, dk, int(terms.window or 0), ctypes.c_float(terms.scale),
-                                               int(splits), _p(part), slopes, sinks, gt, _p(out), _stream()))
+                                               n, nq, nkv, dk, int(terms.window or 0), int(terms.keep_first or 0),
+                                               ctypes.c_float(terms.scale), int(splits), _p(part), slopes, sinks, gt, _p(out),
+                                               _stream()))
     elif fast and k_new is not None and vt_new is not None:
         B = n_cached.shape[0]
         n_tiles = int(sum(-(-int(x) // PREFILL_BLOCK) for x in ctx.host["n_new"]))
@@ -502,8 +501,8 @@ def attention_scored(q, k_new, v_new, pages, nkv: int, dv: int, table, ring_page
         _check(lib().tl_attn_prefill_terms_bf16(_p(q), _p(k_new), _p(vt_new), vt_new.shape[2], _p(ctx.tile_off), _p(pages),
                                                 _p(table), table.shape[1], ring_pages, _p(ctx.row_pos),
                                                 _p(ctx.cu_seqlens), _p(n_cached), B, n_tiles, nq, nkv, dk,
-                                                int(terms.window or 0), ctypes.c_float(terms.scale), slopes, sinks, gt,
-                                                _p(out), _stream()))
+                                                int(terms.window or 0), int(terms.keep_first or 0),
+                                                ctypes.c_float(terms.scale), slopes, sinks, gt, _p(out), _stream()))
     else:
         attn_scored_plain(q, k_new, v_new, pages, nkv, dv, table, ring_pages, ctx.row_seq, ctx.row_pos,
                           ctx.cu_seqlens, n_cached, terms, gate, out)

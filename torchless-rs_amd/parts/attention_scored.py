@@ -228,8 +228,9 @@ def attend_and_commit(ctx, run, q: torch.Tensor, k, v, nkv: int, dk: int, dv: in
     group = run.kv_group
     pages = group.storage[run.kv_layer]
     table = ctx.tables[run.kv_group_index]
-    cores = ops.scored_on_matrix_cores(ctx.dtype, dk, dv) and pages.dim() == 5 and ops.terms_on_matrix_cores(terms)
-    bare = cores and terms.slopes is None and terms.sinks is None and gate is None and att.dtype == ctx.dtype
+    cores = ops.scored_on_matrix_cores(ctx.dtype, dk, dv) and pages.dim() == 5
+    bare = (cores and terms.slopes is None and terms.sinks is None and gate is None and not terms.keep_first
+            and att.dtype == ctx.dtype)
     if ctx.all_single:
         if bare:
             ops.attention(q, None, None, pages, table, group.ring_pages, ctx, ctx.len_after, terms.window, terms.scale, att)
