@@ -103,9 +103,9 @@ ssm_conv_single_kernel(const float* __restrict__ proj, int width, int off, int C
 
 // The recurrence, row after row: one workgroup per (head, sequence, part of the head's columns).  A head's state
 // is kept column by column, S^T [dv, N].  The workgroup takes `dvb` columns; `nsl` neighbouring lanes (a power of
-// two, at most a wave) share a column: lane s keeps rows s, s + nsl, ... of it in registers (R at most) and the
-// column's sum over the rows is a butterfly over those lanes, so a row of the sequence costs no barrier.  The
-// rows' x, B, C, dt' and decay are staged SSM_TB rows at a time.
+// two, at most a wave) share a column: lane s keeps rows s, s + nsl, ... of it in registers (R at most).  The
+// rows' x, B, C, dt' and decay are staged SSM_TB rows at a time; a row of the sequence costs no barrier and no
+// exchange between lanes: the lanes' shares of a column's sum are added once a batch.
 template <typename T, int R>
 __global__ void __launch_bounds__(256)
 ssm_scan_kernel(const T* __restrict__ u, int C, int inner, int G, int N, int heads, int dv, int dvb, int nsl,
@@ -118,6 +118,7 @@ ssm_scan_kernel(const T* __restrict__ u, int C, int inner, int G, int N, int hea
   float* Cs = Bs + SSM_TB * N;         // [SSM_TB][N]
   float* as = Cs + SSM_TB * N;         // [SSM_TB]
   float* dts = as + SSM_TB;            // [SSM_TB]
+  float* part = dts + SSM_TB;          // [SSM_TB][256]: every lane's share of a row's sums
   const int h = blockIdx.x, b = blockIdx.y, d0 = blockIdx.z * dvb;
   const int g = h / (heads / G);
   const int t = threadIdx.x;
@@ -150,35 +151,31 @@ ssm_scan_kernel(const T* __restrict__ u, int C, int inner, int G, int N, int hea
       as[t] = expf(neg_rate * dt);
     }
     __syncthreads();
-    // the batch's rows one after the other, each lane its own rows of the state; the sums over a column's lanes
-    // wait until the batch is through, so that no row waits for a butterfly
-    float sums[SSM_TB];
+    // the batch's rows one after the other, each lane its own rows of the state and no exchange with another: a
+    // lane leaves its share of a row's sum in LDS, and the shares are added after the batch
+#pragma unroll 2
+    for (int i = 0; i < tb; ++i) {
+      const float a = as[i];
+      const float dtx = dts[i] * (active ? xs[i * dvb + dl] : 0.f);
+      float acc = 0.f;
 #pragma unroll
-    for (int i = 0; i < SSM_TB; ++i) {
-      sums[i] = 0.f;
-      if (i < tb) {
-        const float a = as[i];
-        const float dtx = dts[i] * (active ? xs[i * dvb + dl] : 0.f);
-        float acc = 0.f;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          const int nr = s + r * nsl;
-          if (nr < N) {
-            S[r] = fmaf(a, S[r], Bs[i * N + nr] * dtx);
-            acc = fmaf(S[r], Cs[i * N + nr], acc);
-          }
+      for (int r = 0; r < R; ++r) {
+        const int nr = s + r * nsl;
+        if (nr < N) {
+          S[r] = fmaf(a, S[r], Bs[i * N + nr] * dtx);
+          acc = fmaf(S[r], Cs[i * N + nr], acc);
         }
-        sums[i] = acc;
       }
+      part[i * 256 + t] = acc;
     }
-    for (int o = nsl >> 1; o > 0; o >>= 1) {
-#pragma unroll
-      for (int i = 0; i < SSM_TB; ++i) sums[i] += __shfl_xor(sums[i], o, WAVE);
+    __syncthreads();
+    for (int e = t; e < tb * dvb; e += 256) {
+      const int i = e / dvb, c = e % dvb;
+      const float* shares = part + i * 256 + c * nsl;
+      float sum = 0.f;
+      for (int q = 0; q < nsl; ++q) sum += shares[(q + c) & (nsl - 1)];       // (turned by c: neighbours in other banks)
+      y[(size_t)(row0 + i0 + i) * inner + h * dv + d0 + c] = fmaf(skip, xs[i * dvb + c], sum);
     }
-#pragma unroll
-    for (int i = 0; i < SSM_TB; ++i)          // every lane of a column holds the sums: lane s writes rows s, s + nsl, ...
-      if (i < tb && (i & (nsl - 1)) == s && active)
-        y[(size_t)(row0 + i0 + i) * inner + h * dv + d] = fmaf(skip, xs[i * dvb + dl], sums[i]);
   }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
@@ -301,7 +298,7 @@ int tl_ssm_scan(const void* u, int dt, int C, int G, int N, int heads, int dv, c
   TL_REQUIRE(dt == DT_F32 || dt == DT_BF16, "ssm_scan: unknown dtype code %d", dt);
   if (n == 0 || B == 0) return 0;
   const dim3 grid(heads, B, dv / dvb);
-  const size_t lds = sizeof(float) * ((size_t)SSM_TB * (dvb + 2 * N) + 2 * SSM_TB);
+  const size_t lds = sizeof(float) * ((size_t)SSM_TB * (dvb + 2 * N) + 2 * SSM_TB + SSM_TB * 256);
   if (dt == DT_F32)
     scan_launch<float>(R, grid, lds, st, (const float*)u, C, inner, G, N, heads, dv, dvb, nsl, proj, width, dt_off, dt_bias, A_log, D, state, stride,
                        cu_seqlens, slots, y);
