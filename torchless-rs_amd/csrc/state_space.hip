@@ -21,7 +21,7 @@ namespace tl {
 constexpr int SSM_MAX_TAPS = 8;
 constexpr int SSM_MAX_N = 256;
 constexpr int SSM_MAX_DV = 256;
-constexpr int SSM_TB = 16;             // rows of a sequence that the recurrence stages at a time
+constexpr int SSM_TB = 8;              // rows of a sequence that the recurrence stages at a time
 
 __device__ __forceinline__ float silu_f(float a) { return a / (1.0f + expf(-a)); }
 __device__ __forceinline__ float softplus_f(float a) { return fmaxf(a, 0.f) + log1pf(expf(-fabsf(a))); }
@@ -102,76 +102,126 @@ ssm_conv_single_kernel(const float* __restrict__ proj, int width, int off, int C
 }
 
 // The recurrence, row after row: one workgroup per (head, sequence, part of the head's columns).  A head's state
-// is kept column by column, S^T [dv, N].  The workgroup takes `dvb` columns; `nsl` neighbouring lanes (a power of
-// two, at most a wave) share a column: lane s keeps rows s, s + nsl, ... of it in registers (R at most).  The
-// rows' x, B, C, dt' and decay are staged SSM_TB rows at a time; a row of the sequence costs no barrier and no
-// exchange between lanes: the lanes' shares of a column's sum are added once a batch.
-template <typename T, int R>
+// is kept column by column, S^T [dv, N].  The workgroup takes `dvb` columns in groups of DC; `nsl` neighbouring
+// lanes (a power of two, at most a wave) share a group: lane s keeps rows s, s + nsl, ... (R at most) of the
+// group's DC columns in registers, so that a row's B and C are read once for DC columns.  The rows' x, B, C, dt'
+// and decay are staged SSM_TB rows at a time; a row of the sequence costs no barrier and no exchange between
+// lanes: the lanes' shares of a column's sum are left in LDS and added once a batch.
+template <typename T, int R, int DC>
 __global__ void __launch_bounds__(256)
-ssm_scan_kernel(const T* __restrict__ u, int C, int inner, int G, int N, int heads, int dv, int dvb, int nsl,
+ssm_scan_kernel(const T* __restrict__ u, int C, int inner, int G, int N, int heads, int dv, int dvb, int nsl, int NP,
                 const float* __restrict__ proj, int width, int dt_off, const float* __restrict__ dt_bias,
                 const float* __restrict__ A_log, const float* __restrict__ Dw, float* __restrict__ state, long long stride,
                 const int* __restrict__ cu_seqlens, const int* __restrict__ slots, float* __restrict__ y) {
-  extern __shared__ float ssm_lds[];
+  extern __shared__ __attribute__((aligned(16))) float ssm_lds[];
   float* xs = ssm_lds;                 // [SSM_TB][dvb]
-  float* Bs = xs + SSM_TB * dvb;       // [SSM_TB][N]
-  float* Cs = Bs + SSM_TB * N;         // [SSM_TB][N]
-  float* as = Cs + SSM_TB * N;         // [SSM_TB]
+  float* Bs = xs + SSM_TB * dvb;       // [SSM_TB][NP]: NP = R * nsl >= N, zeros behind the N rows, so that the
+  float* Cs = Bs + SSM_TB * NP;        // [SSM_TB][NP]  rows' loop reads without asking where N ends
+  float* as = Cs + SSM_TB * NP;        // [SSM_TB]
   float* dts = as + SSM_TB;            // [SSM_TB]
-  float* part = dts + SSM_TB;          // [SSM_TB][256]: every lane's share of a row's sums
+  float* part = dts + SSM_TB;          // [SSM_TB][dvb][nsl]: every lane's share of a row's sums
   const int h = blockIdx.x, b = blockIdx.y, d0 = blockIdx.z * dvb;
   const int g = h / (heads / G);
   const int t = threadIdx.x;
-  const int s = t % nsl, dl = t / nsl;
-  const bool active = dl < dvb;
-  const int d = d0 + (active ? dl : 0);
+  const int s = t % nsl, cg = t / nsl;
+  const bool active = cg * DC < dvb;
+  const int c0 = active ? cg * DC : 0;                // this lane's first column among the workgroup's
+  const int PW = dvb * nsl;
   const int row0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - row0;
-  float* S_g = state + (long long)slots[b] * stride + (size_t)h * N * dv + (size_t)d * N;
-  float S[R];
+  float* S_g = state + (long long)slots[b] * stride + (size_t)h * N * dv + (size_t)(d0 + c0) * N;
+  float S[R][DC];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int nr = s + r * nsl;
-    S[r] = (active && nr < N) ? S_g[nr] : 0.f;
+#pragma unroll
+    for (int c = 0; c < DC; ++c) S[r][c] = (active && nr < N) ? S_g[(size_t)c * N + nr] : 0.f;
   }
   const float neg_rate = -expf(A_log[h]);
   const float bias = dt_bias[h], skip = Dw[h];
+  // a batch's rows come from memory into registers while the batch before is worked on; which row and column of a
+  // batch a thread fetches is the same for every batch and is worked out once (divisions by sizes that the
+  // compiler does not know)
+  constexpr int XE = SSM_TB * (DC == 1 ? SSM_MAX_DV : 64) / 256, BE = SSM_TB * SSM_MAX_N / 256;
+  int xrow[XE], xcol[XE], brow[BE], boff[BE], blds[BE];
+#pragma unroll
+  for (int k = 0; k < XE; ++k) {
+    const int e = t + 256 * k;
+    xrow[k] = e / dvb;
+    xcol[k] = e % dvb;
+  }
+#pragma unroll
+  for (int k = 0; k < BE; ++k) {
+    const int e = t + 256 * k;
+    brow[k] = e / N;
+    boff[k] = brow[k] * C + inner + g * N + e % N;
+    blds[k] = brow[k] * NP + e % N;
+  }
+  float xr[XE], br[BE], cr[BE], dtr = 0.f;
+  auto load = [&](int i0) {
+    const int tb = min(SSM_TB, n_new - i0);
+    const T* rows = u + (size_t)(row0 + i0) * C;
+#pragma unroll
+    for (int k = 0; k < XE; ++k) xr[k] = xrow[k] < tb ? to_f32(rows[(size_t)xrow[k] * C + h * dv + d0 + xcol[k]]) : 0.f;
+#pragma unroll
+    for (int k = 0; k < BE; ++k) {
+      br[k] = cr[k] = 0.f;
+      if (brow[k] < tb) {
+        br[k] = to_f32(rows[boff[k]]);
+        cr[k] = to_f32(rows[boff[k] + G * N]);
+      }
+    }
+    if (t < tb) dtr = proj[(size_t)(row0 + i0 + t) * width + dt_off + h];
+  };
+  for (int e = t; e < 2 * SSM_TB * NP; e += 256) Bs[e] = 0.f;      // (Bs and Cs lie one behind the other)
+  if (n_new > 0) load(0);
   for (int i0 = 0; i0 < n_new; i0 += SSM_TB) {
     const int tb = min(SSM_TB, n_new - i0);
-    __syncthreads();                     // the last batch's rows have been read
-    for (int e = t; e < tb * dvb; e += 256)
-      xs[e] = to_f32(u[(size_t)(row0 + i0 + e / dvb) * C + h * dv + d0 + e % dvb]);
-    for (int e = t; e < tb * N; e += 256) {
-      const size_t at = (size_t)(row0 + i0 + e / N) * C + inner + g * N + e % N;
-      Bs[e] = to_f32(u[at]);
-      Cs[e] = to_f32(u[at + (size_t)G * N]);
-    }
+    __syncthreads();                     // the last batch's rows and shares have been read
+#pragma unroll
+    for (int k = 0; k < XE; ++k)
+      if (xrow[k] < tb) xs[t + 256 * k] = xr[k];
+#pragma unroll
+    for (int k = 0; k < BE; ++k)
+      if (brow[k] < tb) {
+        Bs[blds[k]] = br[k];
+        Cs[blds[k]] = cr[k];
+      }
     if (t < tb) {
-      const float dt = softplus_f(proj[(size_t)(row0 + i0 + t) * width + dt_off + h] + bias);
+      const float dt = softplus_f(dtr + bias);
       dts[t] = dt;
       as[t] = expf(neg_rate * dt);
     }
     __syncthreads();
-    // the batch's rows one after the other, each lane its own rows of the state and no exchange with another: a
-    // lane leaves its share of a row's sum in LDS, and the shares are added after the batch
+    if (i0 + SSM_TB < n_new) load(i0 + SSM_TB);
 #pragma unroll 2
     for (int i = 0; i < tb; ++i) {
-      const float a = as[i];
-      const float dtx = dts[i] * (active ? xs[i * dvb + dl] : 0.f);
-      float acc = 0.f;
+      const float a = as[i], dt = dts[i];
+      float dtx[DC], acc[DC];
+#pragma unroll
+      for (int c = 0; c < DC; ++c) {
+        dtx[c] = dt * xs[i * dvb + c0 + c];
+        acc[c] = 0.f;
+      }
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        const int nr = s + r * nsl;
-        if (nr < N) {
-          S[r] = fmaf(a, S[r], Bs[i * N + nr] * dtx);
-          acc = fmaf(S[r], Cs[i * N + nr], acc);
+        const float Bv = Bs[i * NP + s + r * nsl], Cv = Cs[i * NP + s + r * nsl];
+#pragma unroll
+        for (int c = 0; c < DC; ++c) {
+          S[r][c] = fmaf(a, S[r][c], Bv * dtx[c]);
+          acc[c] = fmaf(S[r][c], Cv, acc[c]);
         }
       }
-      part[i * 256 + t] = acc;
+      if (active) {
+#pragma unroll
+        for (int c = 0; c < DC; ++c) part[i * PW + (c0 + c) * nsl + s] = acc[c];
+      }
     }
     __syncthreads();
-    for (int e = t; e < tb * dvb; e += 256) {
-      const int i = e / dvb, c = e % dvb;
-      const float* shares = part + i * 256 + c * nsl;
+#pragma unroll
+    for (int k = 0; k < XE; ++k) {
+      if (xrow[k] >= tb) break;
+      const int i = xrow[k], c = xcol[k];
+      const float* shares = part + i * PW + c * nsl;
       float sum = 0.f;
       for (int q = 0; q < nsl; ++q) sum += shares[(q + c) & (nsl - 1)];       // (turned by c: neighbours in other banks)
       y[(size_t)(row0 + i0 + i) * inner + h * dv + d0 + c] = fmaf(skip, xs[i * dvb + c], sum);
@@ -180,7 +230,9 @@ ssm_scan_kernel(const T* __restrict__ u, int C, int inner, int G, int N, int hea
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int nr = s + r * nsl;
-    if (active && nr < N) S_g[nr] = S[r];
+#pragma unroll
+    for (int c = 0; c < DC; ++c)
+      if (active && nr < N) S_g[(size_t)c * N + nr] = S[r][c];
   }
 }
 
@@ -211,33 +263,61 @@ ssm_gate_norm_kernel(const float* __restrict__ y, const float* __restrict__ proj
 
 using namespace tl;
 
-template <typename T>
-static int scan_launch(int R, dim3 grid, size_t lds, hipStream_t st, const T* u, int C, int inner, int G, int N, int heads, int dv, int dvb,
-                       int nsl, const float* proj, int width, int dt_off, const float* dt_bias, const float* A_log, const float* D,
-                       float* state, long long stride, const int* cu, const int* slots, float* y) {
-#define TL_SCAN(RR)                                                                                                       \
-  ssm_scan_kernel<T, RR><<<grid, 256, lds, st>>>(u, C, inner, G, N, heads, dv, dvb, nsl, proj, width, dt_off, dt_bias, A_log, D, \
-                                               state, stride, cu, slots, y)
-  if (R <= 4) TL_SCAN(4);
-  else if (R <= 8) TL_SCAN(8);
-  else if (R <= 16) TL_SCAN(16);
-  else if (R <= 32) TL_SCAN(32);
-  else TL_SCAN(64);
-#undef TL_SCAN
-  return 0;
-}
-
-// How a head's dv columns are cut over workgroups and a workgroup's 256 lanes over its columns.
-static void scan_shape(int N, int dv, int& dvb, int& nsl, int& R) {
-  dvb = dv;                                   // the largest part of dv of at most 16 columns, if it has one of 4 or more
-  for (int c = 16; c >= 4; --c)
-    if (dv % c == 0) {
-      dvb = c;
+// How a head's dv columns are cut over workgroups and a workgroup's 256 lanes over its columns: lanes take DC = 4
+// columns each where dv allows it, a workgroup the largest part of dv of at most `most` columns (a multiple of DC).
+struct ScanShape {
+  int DC, dvb, nsl, R;
+};
+static ScanShape scan_shape_for(int N, int dv, int DC, int most) {
+  ScanShape z{DC, dv, 1, 0};
+  for (int c = most; c >= DC; c -= DC)
+    if (c % DC == 0 && dv % c == 0) {
+      z.dvb = c;
       break;
     }
-  nsl = 1;
-  while (nsl * 2 <= WAVE && nsl * 2 * dvb <= 256 && nsl < N) nsl *= 2;
-  R = (N + nsl - 1) / nsl;
+  const int groups = z.dvb / DC;
+  while (z.nsl * 2 <= WAVE && z.nsl * 2 * groups <= 256 && z.nsl < N) z.nsl *= 2;
+  z.R = (N + z.nsl - 1) / z.nsl;
+  return z;
+}
+// `units`: heads x sequences.  Few of them take fewer columns a workgroup (down to 16), so that the device's
+// compute units all have work; many take up to 64, so that a row's B and C are staged for more columns at once.
+static ScanShape scan_shape(int N, int dv, int units) {
+  if (dv % 4 == 0) {
+    ScanShape best{};
+    for (int most = 64; most >= 16; most /= 2) {
+      const ScanShape z = scan_shape_for(N, dv, 4, most);
+      if (z.R > 16) continue;
+      best = z;
+      if ((long long)units * (dv / z.dvb) >= 512) break;
+    }
+    if (best.DC == 4) return best;
+  }
+  return scan_shape_for(N, dv, 1, 64);
+}
+
+template <typename T>
+static int scan_launch(const ScanShape& z, dim3 grid, size_t lds, hipStream_t st, const T* u, int C, int inner, int G, int N,
+                       int heads, int dv, const float* proj, int width, int dt_off, const float* dt_bias, const float* A_log,
+                       const float* D, float* state, long long stride, const int* cu, const int* slots, float* y) {
+#define TL_SCAN(RR, DD)                                                                                                      \
+  ssm_scan_kernel<T, RR, DD><<<grid, 256, lds, st>>>(u, C, inner, G, N, heads, dv, z.dvb, z.nsl, RR * z.nsl, proj, width, dt_off, dt_bias, \
+                                                     A_log, D, state, stride, cu, slots, y)
+  if (z.DC == 4) {
+    if (z.R <= 1) TL_SCAN(1, 4);
+    else if (z.R <= 2) TL_SCAN(2, 4);
+    else if (z.R <= 4) TL_SCAN(4, 4);
+    else if (z.R <= 8) TL_SCAN(8, 4);
+    else TL_SCAN(16, 4);
+  } else {
+    if (z.R <= 4) TL_SCAN(4, 1);
+    else if (z.R <= 8) TL_SCAN(8, 1);
+    else if (z.R <= 16) TL_SCAN(16, 1);
+    else if (z.R <= 32) TL_SCAN(32, 1);
+    else TL_SCAN(64, 1);
+  }
+#undef TL_SCAN
+  return 0;
 }
 
 extern "C" {
@@ -290,20 +370,21 @@ int tl_ssm_scan(const void* u, int dt, int C, int G, int N, int heads, int dv, c
   const int inner = heads * dv;
   TL_REQUIRE(C == inner + 2 * G * N && dt_off >= 0 && dt_off + heads <= width, "ssm_scan: %d channels for heads=%d dv=%d G=%d N=%d", C,
              heads, dv, G, N);
-  int dvb, nsl, R;
-  scan_shape(N, dv, dvb, nsl, R);
-  TL_REQUIRE(R <= 64, "ssm_scan: a state of %d x %d gives a thread %d rows (at most 64)", N, dv, R);
+  const ScanShape z = scan_shape(N, dv, heads * B);
+  TL_REQUIRE(z.R <= 64, "ssm_scan: a state of %d x %d gives a thread %d rows (at most 64)", N, dv, z.R);
   TL_REQUIRE(stride >= (long long)heads * N * dv, "ssm_scan: a sequence's block is too small");
   TL_REQUIRE(u && proj && dt_bias && A_log && D && state && cu_seqlens && slots && y, "ssm_scan: a buffer is missing");
   TL_REQUIRE(dt == DT_F32 || dt == DT_BF16, "ssm_scan: unknown dtype code %d", dt);
   if (n == 0 || B == 0) return 0;
-  const dim3 grid(heads, B, dv / dvb);
-  const size_t lds = sizeof(float) * ((size_t)SSM_TB * (dvb + 2 * N) + 2 * SSM_TB + SSM_TB * 256);
+  const dim3 grid(heads, B, dv / z.dvb);
+  int Rt = z.DC == 4 ? 1 : 4;                          // the rows of the kernel that `scan_launch` picks
+  while (Rt < z.R) Rt *= 2;
+  const size_t lds = sizeof(float) * ((size_t)SSM_TB * (z.dvb + 2 * Rt * z.nsl) + 2 * SSM_TB + (size_t)SSM_TB * z.dvb * z.nsl);
   if (dt == DT_F32)
-    scan_launch<float>(R, grid, lds, st, (const float*)u, C, inner, G, N, heads, dv, dvb, nsl, proj, width, dt_off, dt_bias, A_log, D, state, stride,
+    scan_launch<float>(z, grid, lds, st, (const float*)u, C, inner, G, N, heads, dv, proj, width, dt_off, dt_bias, A_log, D, state, stride,
                        cu_seqlens, slots, y);
   else
-    scan_launch<bf16>(R, grid, lds, st, (const bf16*)u, C, inner, G, N, heads, dv, dvb, nsl, proj, width, dt_off, dt_bias, A_log, D, state, stride,
+    scan_launch<bf16>(z, grid, lds, st, (const bf16*)u, C, inner, G, N, heads, dv, proj, width, dt_off, dt_bias, A_log, D, state, stride,
                       cu_seqlens, slots, y);
   TL_LAUNCH_CHECK("ssm_scan");
   return 0;
