@@ -651,6 +651,32 @@ def test_logits_do_not_depend_on_batch_mates(zoo, dtype):
     assert rel_err(lg[:len(p)][sure], alone[sure]) < (1e-6 if dtype == "float32" else 2e-2)
 
 
+def test_many_rows_run_expert_by_expert(zoo, monkeypatch):
+    """A prompt of more rows than the framework's own products take, with the bar for sorting rows by expert taken
+    down to the tests' sizes: the same logits from every expert's products over its own rows alone."""
+    from torchless_rs_amd.engine import SeqInput
+    from torchless_rs_amd.parts import ffn_routed
+    monkeypatch.setattr(ffn_routed, "GROUPED_ROWS_PER_EXPERT", 1)
+    calls = []
+    inner = ffn_routed.RoutedExperts._grouped
+    monkeypatch.setattr(ffn_routed.RoutedExperts, "_grouped", lambda self, *a: (calls.append(a[1].shape[0]), inner(self, *a))[1])
+    for name in ("cores", "mixed"):
+        eng, z = engine_for(zoo, name, "bfloat16"), zoo[name]
+        p = z["prompts"][3]
+        calls.clear()
+        s = eng.alloc()
+        got = eng.step([SeqInput(s, p, list(range(len(p))))]).clone()
+        eng.free(s)
+        assert calls and all(c == len(p) for c in calls), calls
+        close(got, z["want"][3], "bfloat16", (name, "expert by expert"), z["margin"][3])
+        s = eng.alloc()                                                   # two unequal prompts in one step
+        q = z["prompts"][2]
+        got = eng.step([SeqInput(s, p, [len(p) - 1]), SeqInput(eng.alloc(), q, list(range(len(q))))]).clone()
+        for h in eng.cache.held_slots():
+            eng.free(h)
+        close(got[1:], z["want"][2], "bfloat16", (name, "expert by expert, two prompts"), z["margin"][2])
+
+
 def test_greedy_generation_through_the_entry_point(zoo):
     from torchless_rs_amd import SamplingConfig, generate_until_eos
     for name in ("mixed", "ones", "odd"):

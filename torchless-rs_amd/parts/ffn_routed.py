@@ -17,6 +17,12 @@ products of the framework's own kinds and no gather or scatter, whatever the tok
 reads every expert's weights in every step, as a step of many rows does anyway, and multiplies
 `n_experts / top` times what the chosen experts alone would.
 
+A step of many rows in bfloat16 (on average `GROUPED_ROWS_PER_EXPERT` rows an expert or more, more rows
+than the framework's own product kernels take, so that no graph holds the step) sorts the
+(row, chosen expert) pairs by expert and runs every expert's two products over its own rows
+(`_grouped`): the chosen experts' multiplications alone, at the price of one count per expert
+read back by the host.
+
 A step of few rows (rows * top <= n_experts: the rows cannot use every expert) runs the chosen
 experts alone: per row two products of its experts' matrices with a vector
 (`ops.expert_rows_up`, `ops.expert_rows_down`), which read `top` experts' weights a row and
@@ -33,6 +39,9 @@ from ..kernels import ops
 from ..weights.binding import WeightSpec
 from .base import FeedForward, flush_pending, register_part
 from .linear import Linear
+
+
+GROUPED_ROWS_PER_EXPERT = 128      # from this many rows an expert on average, experts run over their own rows
 
 
 class PlainFeedForward(FeedForward):
@@ -144,6 +153,54 @@ class RoutedExperts(FeedForward):
         ops.expert_rows_up(y, self.up.weight, chosen, weights, self.ff, self.shared, self.activation, hs)
         ops.expert_rows_down(hs, self.down.weight, chosen, self.E, self.ff, self.shared, out, accumulate)
 
+    def many_rows(self, ctx, y: torch.Tensor) -> bool:
+        """Do the rows of `y` run expert by expert over each expert's own rows?"""
+        n = y.shape[0]
+        return (y.dtype == torch.bfloat16 and self.up.weight.dtype == self.down.weight.dtype == torch.bfloat16
+                and n * self.top >= GROUPED_ROWS_PER_EXPERT * self.E and not self.up.own_kernels(n)
+                and not ctx.host.get("fixed_launches"))
+
+    def _grouped(self, ctx, y: torch.Tensor, out: torch.Tensor, accumulate: bool) -> None:
+        n, E, top, ff, H = y.shape[0], self.E, self.top, self.ff, self.H
+        ws = ctx.workspace
+        weights = ws.get("experts_w", (n, E), torch.float32)
+        chosen = ws.get("experts_chosen", (n, top), torch.int32)
+        ops.route(y, self.router, self.groups, self.keep, self.top, weights, chosen)
+        flat = chosen.view(-1).long()
+        order = torch.argsort(flat, stable=True)                       # pairs by expert, a row's place kept within one
+        counts = torch.bincount(flat, minlength=E).tolist()            # (the host waits for the router here)
+        rows = torch.div(order, top, rounding_mode="floor")
+        ys = y.index_select(0, rows)                                   # [n * top, H]
+        scale = weights.gather(1, chosen.long()).view(-1).index_select(0, order).view(-1, 1).contiguous()
+        up_w, down_w = self.up.weight, self.down.weight
+        u = ws.get("experts_gu", (n * top, ff), torch.float32)
+        at = 0
+        for e, c in enumerate(counts):
+            if c:
+                ops.gemm(ys[at:at + c], up_w[e * ff:(e + 1) * ff], u[at:at + c])
+                at += c
+        h = ws.get("experts_gh", (n * top, ff), y.dtype)
+        ops.expert_act(u, scale, 1, ff, self.activation, h)
+        z = ws.get("experts_gz", (n * top, H), torch.float32)
+        at = 0
+        for e, c in enumerate(counts):
+            if c:
+                torch.mm(h[at:at + c], down_w[:, e * ff:(e + 1) * ff].t(), out_dtype=torch.float32, out=z[at:at + c])
+                at += c
+        back = torch.empty_like(order)
+        back[order] = torch.arange(n * top, device=order.device)
+        total = z.index_select(0, back).view(n, top, H).sum(dim=1)     # a row's experts in the order it chose them
+        if self.shared:
+            us = ws.get("experts_su", (n, self.shared), torch.float32)
+            ops.gemm(y, up_w[E * ff:], us)
+            hs = ws.get("experts_sh", (n, self.shared), y.dtype)
+            ops.expert_act(us, None, 0, self.shared, self.activation, hs)
+            total.add_(torch.mm(hs, down_w[:, E * ff:].t(), out_dtype=torch.float32))
+        if accumulate:
+            out.add_(total)
+        else:
+            out.copy_(total)
+
     def _hidden(self, ctx, y: torch.Tensor) -> torch.Tensor:
         n = y.shape[0]
         ws = ctx.workspace
@@ -160,11 +217,18 @@ class RoutedExperts(FeedForward):
             flush_pending(ctx, x)
             self._rows(ctx, y, x, True)
             return
+        if self.many_rows(ctx, y):
+            flush_pending(ctx, x)
+            self._grouped(ctx, y, x, True)
+            return
         self.down.add_into(self._hidden(ctx, y), x, ctx, "experts_down_parts")
 
     def produce(self, ctx, y: torch.Tensor, out: torch.Tensor) -> None:
         if self.few_rows(y):
             self._rows(ctx, y, out, False)
+            return
+        if self.many_rows(ctx, y):
+            self._grouped(ctx, y, out, False)
             return
         self.down(self._hidden(ctx, y), out)
 
