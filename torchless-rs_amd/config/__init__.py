@@ -4,7 +4,8 @@ from .base import (ArchitectureEntry, ConfigError, ModelConfig, architecture_nam
 from .mistral import MistralConfig
 from .sozetar import SozetarConfig
 from .fanitar import FanitarConfig
+from .nepisun import NepisunConfig
 
-__all__ = ["ArchitectureEntry", "ConfigError", "ModelConfig", "MistralConfig", "SozetarConfig", "FanitarConfig", "architecture_name",
+__all__ = ["ArchitectureEntry", "ConfigError", "ModelConfig", "MistralConfig", "SozetarConfig", "FanitarConfig", "NepisunConfig", "architecture_name",
            "config_from_dict", "get_architecture", "load_config", "register_architecture",
            "registered_architectures", "unregister_architecture"]
