@@ -20,7 +20,7 @@ constexpr int RT_MAX_E = 1024;
 template <typename T>
 __global__ void __launch_bounds__(256)
 route_kernel(const T* __restrict__ h, int W, const float* __restrict__ wr, int E, int groups, int keep, int top,
-             float* __restrict__ weights, int* __restrict__ chosen) {
+             float* __restrict__ weights, int* __restrict__ chosen, bool vec) {
   __shared__ float s_s[RT_MAX_E];
   __shared__ float g_s[RT_MAX_E];
   __shared__ unsigned char ok_s[RT_MAX_E];
@@ -31,14 +31,27 @@ route_kernel(const T* __restrict__ h, int W, const float* __restrict__ wr, int E
   for (int e = wave; e < E; e += 4) {
     const float* w = wr + (size_t)e * W;
     float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;      // four chains: the loads of one do not wait for another's sum
-    int c = lane;
-    for (; c + 3 * WAVE < W; c += 4 * WAVE) {
-      d0 = fmaf(w[c], to_f32(row[c]), d0);
-      d1 = fmaf(w[c + WAVE], to_f32(row[c + WAVE]), d1);
-      d2 = fmaf(w[c + 2 * WAVE], to_f32(row[c + 2 * WAVE]), d2);
-      d3 = fmaf(w[c + 3 * WAVE], to_f32(row[c + 3 * WAVE]), d3);
+    int c = 0;
+    if (vec) {                                         // four channels a lane and load
+#pragma unroll 4
+      for (c = lane * 4; c + 3 < W; c += WAVE * 4) {
+        const f32x4 wv = *reinterpret_cast<const f32x4*>(w + c);
+        float r0, r1, r2, r3;
+        if constexpr (sizeof(T) == 2) {
+          const bf16x4 rv = *reinterpret_cast<const bf16x4*>(row + c);
+          r0 = (float)rv[0], r1 = (float)rv[1], r2 = (float)rv[2], r3 = (float)rv[3];
+        } else {
+          const f32x4 rv = *reinterpret_cast<const f32x4*>(row + c);
+          r0 = rv[0], r1 = rv[1], r2 = rv[2], r3 = rv[3];
+        }
+        d0 = fmaf(wv[0], r0, d0);
+        d1 = fmaf(wv[1], r1, d1);
+        d2 = fmaf(wv[2], r2, d2);
+        d3 = fmaf(wv[3], r3, d3);
+      }
+    } else {
+      for (c = lane; c < W; c += WAVE) d0 = fmaf(w[c], to_f32(row[c]), d0);
     }
-    for (; c < W; c += WAVE) d0 = fmaf(w[c], to_f32(row[c]), d0);
     float dot = wave_sum((d0 + d1) + (d2 + d3));
     if (lane == 0) s_s[e] = dot;
   }
@@ -208,10 +221,11 @@ int tl_route(const void* h, int dt, int n, int W, const float* wr, int E, int gr
              "route: %d experts in %d groups of which %d are kept cannot give %d", E, groups, keep, top);
   TL_REQUIRE(h && wr && weights, "route: a buffer is missing");
   if (n == 0) return 0;
+  const bool vec = W % 4 == 0 && (uintptr_t)h % 16 == 0 && (uintptr_t)wr % 16 == 0;
   if (dt == DT_F32)
-    route_kernel<float><<<n, 256, 0, st>>>((const float*)h, W, wr, E, groups, keep, top, weights, chosen);
+    route_kernel<float><<<n, 256, 0, st>>>((const float*)h, W, wr, E, groups, keep, top, weights, chosen, vec);
   else if (dt == DT_BF16)
-    route_kernel<bf16><<<n, 256, 0, st>>>((const bf16*)h, W, wr, E, groups, keep, top, weights, chosen);
+    route_kernel<bf16><<<n, 256, 0, st>>>((const bf16*)h, W, wr, E, groups, keep, top, weights, chosen, vec);
   else
     TL_REQUIRE(false, "route: unknown dtype code %d", dt);
   TL_LAUNCH_CHECK("route");
