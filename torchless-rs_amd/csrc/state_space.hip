@@ -222,8 +222,18 @@ ssm_scan_kernel(const T* __restrict__ u, int C, int inner, int G, int N, int hea
       if (xrow[k] >= tb) break;
       const int i = xrow[k], c = xcol[k];
       const float* shares = part + i * PW + c * nsl;
+      // (turned by c: neighbours in other banks; eight sums at a time: a load does not wait for the one before)
       float sum = 0.f;
-      for (int q = 0; q < nsl; ++q) sum += shares[(q + c) & (nsl - 1)];       // (turned by c: neighbours in other banks)
+      if (nsl >= 8) {
+        float p[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int q = 0; q < nsl; q += 8) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) p[j] += shares[(q + j + c) & (nsl - 1)];
+        }
+        sum = ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
+      } else {
+        for (int q = 0; q < nsl; ++q) sum += shares[(q + c) & (nsl - 1)];
+      }
       y[(size_t)(row0 + i0 + i) * inner + h * dv + d0 + c] = fmaf(skip, xs[i * dvb + c], sum);
     }
   }
