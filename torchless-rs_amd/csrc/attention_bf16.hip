@@ -45,6 +45,13 @@ struct MoreTerms {
   const float* gate;
   int keep_first;          // with a window: positions 0 .. keep_first - 1 stay visible beside it (the cache then keeps
                            // every position: no ring of pages)
+  int chunk;               // > 0: a key is seen only inside the query's run of `chunk` positions counted from the
+                           // sequence's start, floor(j / chunk) == floor(p / chunk)
+  int logistic;            // the LOGI variants: a key's weight is 1 / (1 + exp(-(score + score_bias[h]))), every key by
+                           // itself, no normalisation.  In the kernels' terms: the running maximum stays at 0, the sum
+                           // holds nothing but a 1 (as a sink of score 0 would leave it, once a row), so that splits
+                           // and their merge work unchanged and the final division is one by 1
+  const float* score_bias; // [nq] or null
 };
 
 // The pages that a query at p reads, numbered 0 .. n - 1 in the order they are read: the pages of the window
@@ -70,7 +77,7 @@ struct PageSpan {
 constexpr int PF_BM = 128, PF_BN = 64, PF_VLD = PF_BN + 4;
 constexpr int PF_PART_HEAD = 4;       // floats before O in a half block's partial result: maximum, sum, two of padding
 
-template <int DPAD, bool LEAN, bool TERMS = false>   // LEAN (d == DPAD, 256 % (DPAD / 8) == 0): whole tiles are fetched the short way
+template <int DPAD, bool LEAN, bool TERMS = false, bool LOGI = false>   // LEAN (d == DPAD, 256 % (DPAD / 8) == 0): whole tiles are fetched the short way
 __global__ void __launch_bounds__(256, DPAD <= 128 ? 2 : 1)
 attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
                     const bf16* __restrict__ vt_new, int vt_cols, const int* __restrict__ tile_off,
@@ -170,11 +177,21 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
     }
     if (terms.slopes != nullptr) slope = terms.slopes[h];
   }
+  float sbias = 0.f;
+  if constexpr (LOGI) {
+    static_assert(TERMS, "logistic weights are a variant of the kernel with terms");
+    m = 0.f;
+    l = 1.f;
+    if (terms.score_bias != nullptr) sbias = terms.score_bias[h];
+  }
+  const int chunk = TERMS ? terms.chunk : 0;
   const float sc = TERMS ? 1.f : scale;       // with TERMS the scores are scaled where the bias is added
 
   const int p_lo = p_first + qt0, p_hi = p_first + min(qt0 + PF_BM, n_new) - 1;
   const int pw_lo = p_lo + wave * 32, pw_hi = min(p_hi, pw_lo + 31);    // this wave's positions
-  const int j_lo = (window > 0 && p_lo - window + 1 > 0) ? p_lo - window + 1 : 0;
+  int j_lo = (window > 0 && p_lo - window + 1 > 0) ? p_lo - window + 1 : 0;
+  if (chunk > 0) j_lo = max(j_lo, (p_lo / chunk) * chunk);
+  const int c_lo_me = chunk > 0 ? (p_me / chunk) * chunk : 0;         // the first key of this lane's query's chunk
 
   bf16x8 kfetch[PT], vfetch[PT];
   // tile j0 -> registers: keys as rows [key][d], values as rows [dv][key]
@@ -316,6 +333,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
     }
     // does any query of this wave see any key of this tile?
     if (pw_lo > p_hi || j0 > pw_hi || (window > 0 && j0 + PF_BN - 1 <= pw_lo - window && j0 >= keep)) continue;
+    if (chunk > 0 && j0 + PF_BN - 1 < (pw_lo / chunk) * chunk) continue;       // before every chunk of the wave's queries
 
     f32x16 s[2];
 #pragma unroll
@@ -339,47 +357,52 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int j = j0 + nb * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-          s[nb][r] = s[nb][r] * scale - slope * (float)(p_me - j);
+          s[nb][r] = s[nb][r] * scale - slope * (float)(p_me - j) + sbias;
         }
     }
     const bool edge = j0 + PF_BN - 1 > pw_lo || (window > 0 && j0 <= pw_hi - window) ||
-                      pw_lo + 31 > pw_hi;
+                      pw_lo + 31 > pw_hi || (chunk > 0 && j0 < (pw_hi / chunk) * chunk);
     if (edge) {
 #pragma unroll
       for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int j = j0 + nb * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-          const bool ok = q_ok && j <= p_me && (window == 0 || j > p_me - window || j < keep);
+          const bool ok = q_ok && j <= p_me && (window == 0 || j > p_me - window || j < keep) && j >= c_lo_me;
           s[nb][r] = ok ? s[nb][r] : -INFINITY;
         }
     }
-    float tmax = -INFINITY;
+    float c1 = -1.44269504088896f, c0 = 0.f;             // (logistic weights: 1 / (1 + 2^(s * c1)))
+    if constexpr (!LOGI) {
+      float tmax = -INFINITY;
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb)
+      for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[nb][r]);
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
-    const float m_new = fmaxf(m, tmax * sc);             // scale > 0: the maximum of the scaled scores
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    if (__ballot(m_new != m) != 0ull) {                  // the running maximum moved in some lane
-      const float alpha = __expf(m - m_use);
-      l *= alpha;
+        for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[nb][r]);
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+      const float m_new = fmaxf(m, tmax * sc);             // scale > 0: the maximum of the scaled scores
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      if (__ballot(m_new != m) != 0ull) {                  // the running maximum moved in some lane
+        const float alpha = __expf(m - m_use);
+        l *= alpha;
 #pragma unroll
-      for (int vb = 0; vb < VB; ++vb)
+        for (int vb = 0; vb < VB; ++vb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o[vb][r] *= alpha;
-      m = m_new;
+          for (int r = 0; r < 16; ++r) o[vb][r] *= alpha;
+        m = m_new;
+      }
+      // p = exp(s * scale - m) = 2^(s * c1 + c0)
+      c1 = sc * 1.44269504088896f;
+      c0 = -m_use * 1.44269504088896f;
     }
-    // p = exp(s * scale - m) = 2^(s * c1 + c0)
-    const float c1 = sc * 1.44269504088896f, c0 = -m_use * 1.44269504088896f;
     float psum = 0.f;
     bf16x8 pb[2][2];
     bf16x8 pb_lo[TERMS ? 2 : 1][2];       // what the rounding of a weight to bfloat16 left over
     // probability e of the tile's 32 (e = 16 nb + r), in the order of the sum
     auto soft = [&](int e) {
       const int nb = e / 16, r = e % 16;
-      const float pv = __builtin_amdgcn_exp2f(fmaf(s[nb][r], c1, c0));
+      float pv = __builtin_amdgcn_exp2f(fmaf(s[nb][r], c1, c0));
+      if constexpr (LOGI) pv = __builtin_amdgcn_rcpf(1.0f + pv);      // a masked key: 2^inf, weight 0
       psum += pv;
       const bf16 hi = (bf16)pv;
       pb[nb][r / 8][r % 8] = hi;
@@ -423,7 +446,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
     }
     __builtin_amdgcn_s_setprio(0);
     psum += __shfl_xor(psum, 32, WAVE);
-    l += psum;
+    if constexpr (!LOGI) l += psum;
   }
   if (ways != 0) {
     // a run of a block's keys: running maximum, sum and unscaled O of every row, for the merge
@@ -508,7 +531,7 @@ attn_prefill_merge_kernel(const float* __restrict__ part, int part_ways, const i
 // result is written at once.
 constexpr int DC_WAVES = 4;
 
-template <int DPAD, bool LEAN, bool TERMS = false>   // DPAD: multiple of 32; LEAN: d == DPAD, loads without guards at fixed offsets
+template <int DPAD, bool LEAN, bool TERMS = false, bool LOGI = false>   // DPAD: multiple of 32; LEAN: d == DPAD, loads without guards at fixed offsets
 __global__ void __launch_bounds__(DC_WAVES * 64)
 attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
                    const int* __restrict__ table, int table_stride, int ring_pages,
@@ -528,7 +551,8 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
   const int hl = hg * 16 + li;                        // head within the KV group (column of S^T)
   const int h = kvh * g + min(hl, g - 1);
   const int p = row_pos[b];
-  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  if (TERMS && terms.chunk > 0) lo = max(lo, (p / terms.chunk) * terms.chunk);
   const int keep = (TERMS && window > 0) ? terms.keep_first : 0;
   const PageSpan span(lo, p, keep);
   // [my_lo, my_hi): the pages (as the span numbers them) in shares that differ by one at most (65 pages in 8
@@ -549,10 +573,12 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
   f32x4 o[VB];
 #pragma unroll
   for (int vb = 0; vb < VB; ++vb) o[vb] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, l = 0.f;
-  float slope = 0.f;
+  float m = LOGI ? 0.f : -INFINITY, l = 0.f;
+  float slope = 0.f, sbias = 0.f;
   if constexpr (TERMS)
     if (terms.slopes != nullptr) slope = terms.slopes[h];
+  if constexpr (LOGI)
+    if (terms.score_bias != nullptr) sbias = terms.score_bias[h];
 
   // the split's groups of 32 keys go round the waves; a wave's pages are two apart, and the id of
   // its next page is looked up while it works on this one
@@ -623,26 +649,26 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
       for (int e = 0; e < 8; ++e) {
         const int j = j0 + 8 * kg + e;
         const bool ok = j <= p && (j >= lo || j < keep);
-        if constexpr (TERMS) sv[e] = ok ? s[e / 4][e % 4] * scale - slope * (float)(p - j) : -INFINITY;
+        if constexpr (TERMS) sv[e] = ok ? s[e / 4][e % 4] * scale - slope * (float)(p - j) + sbias : -INFINITY;
         else sv[e] = ok ? s[e / 4][e % 4] * scale : -INFINITY;
         tmax = fmaxf(tmax, sv[e]);
       }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
-      const float m_new = fmaxf(m, tmax);              // finite: the group holds a visible key
-      const float alpha = __expf(m - m_new);
+      const float m_new = LOGI ? 0.f : fmaxf(m, tmax);  // finite: the group holds a visible key
+      const float alpha = LOGI ? 1.f : __expf(m - m_new);
       float psum = 0.f;
       bf16x8 pb, pb_lo;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float pv = __expf(sv[e] - m_new);
+        const float pv = LOGI ? 1.0f / (1.0f + __expf(-sv[e])) : __expf(sv[e] - m_new);
         psum += pv;
         pb[e] = (bf16)pv;
         if constexpr (TERMS) pb_lo[e] = (bf16)(pv - (float)pb[e]);
       }
       psum += __shfl_xor(psum, 16, WAVE);
       psum += __shfl_xor(psum, 32, WAVE);
-      l = l * alpha + psum;
+      if constexpr (!LOGI) l = l * alpha + psum;
       m = m_new;
       // O^T[dv][head] += V^T[dv][keys] P^T[keys][head]; values lie as [d][PAGE] in the page
       if (j0 + 31 > p) {           // rows past the sequence's end were never written: 0 * garbage
@@ -732,6 +758,7 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
         mh = ms;
       }
     }
+    if constexpr (LOGI) ll = split == 0 ? 1.f : 0.f;    // the sum is a 1, once for a row
     if (n_splits == 1) {                                // nothing to merge with
       float res = o_sum(idx) * fs / ll;
       if constexpr (TERMS)
@@ -766,7 +793,7 @@ template <int N> __device__ __forceinline__ void wait_page_loads_but() {     // 
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-template <int D, int NS, bool TERMS = false>
+template <int D, int NS, bool TERMS = false, bool LOGI = false>
 __global__ void __launch_bounds__(DC_WAVES * 64)
 attn_decode_ring_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
                         const int* __restrict__ table, int table_stride, int ring_pages,
@@ -791,7 +818,8 @@ attn_decode_ring_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pag
   const int hl = hg * 16 + li;
   const int h = kvh * g + min(hl, g - 1);
   const int p = row_pos[b];
-  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  if (TERMS && terms.chunk > 0) lo = max(lo, (p / terms.chunk) * terms.chunk);
   const int keep = (TERMS && window > 0) ? terms.keep_first : 0;
   const PageSpan span(lo, p, keep);
   const int my_lo = (int)((long long)split * span.n / n_splits);
@@ -841,10 +869,12 @@ attn_decode_ring_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pag
   f32x4 o[VB];
 #pragma unroll
   for (int vb = 0; vb < VB; ++vb) o[vb] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, l = 0.f;
-  float slope = 0.f;
+  float m = LOGI ? 0.f : -INFINITY, l = 0.f;
+  float slope = 0.f, sbias = 0.f;
   if constexpr (TERMS)
     if (terms.slopes != nullptr) slope = terms.slopes[h];
+  if constexpr (LOGI)
+    if (terms.score_bias != nullptr) sbias = terms.score_bias[h];
 
 #pragma unroll
   for (int st = 0; st < NS - 1; ++st)
@@ -878,26 +908,26 @@ attn_decode_ring_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pag
     for (int r = 0; r < 4; ++r) {
       const int j = j0 + 4 * kg + r;
       const bool ok = j <= p && (j >= lo || j < keep);
-      if constexpr (TERMS) sv[r] = ok ? s[r] * scale - slope * (float)(p - j) : -INFINITY;
+      if constexpr (TERMS) sv[r] = ok ? s[r] * scale - slope * (float)(p - j) + sbias : -INFINITY;
       else sv[r] = ok ? s[r] * scale : -INFINITY;
       tmax = fmaxf(tmax, sv[r]);
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
-    const float m_new = fmaxf(m, tmax);               // finite: one of the 16 keys is visible
-    const float alpha = __expf(m - m_new);
+    const float m_new = LOGI ? 0.f : fmaxf(m, tmax);  // finite: one of the 16 keys is visible
+    const float alpha = LOGI ? 1.f : __expf(m - m_new);
     float psum = 0.f;
     bf16x4 pb, pb_lo;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const float pv = __expf(sv[r] - m_new);
+      const float pv = LOGI ? 1.0f / (1.0f + __expf(-sv[r])) : __expf(sv[r] - m_new);
       psum += pv;
       pb[r] = (bf16)pv;
       if constexpr (TERMS) pb_lo[r] = (bf16)(pv - (float)pb[r]);
     }
     psum += __shfl_xor(psum, 16, WAVE);
     psum += __shfl_xor(psum, 32, WAVE);
-    l = l * alpha + psum;
+    if constexpr (!LOGI) l = l * alpha + psum;
     m = m_new;
     if (j0 + 15 > p) {                                // rows past the sequence's end were never written: 0 * garbage
       typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
@@ -970,6 +1000,7 @@ attn_decode_ring_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pag
         mh = ms;
       }
     }
+    if constexpr (LOGI) ll = split == 0 ? 1.f : 0.f;  // the sum is a 1, once for a row
     if (n_splits == 1) {
       float res = osum / ll;
       if constexpr (TERMS)
@@ -1040,7 +1071,7 @@ attn_decode_combine_kernel(const float* __restrict__ part, int n_splits, int d, 
     if (lane + 64 * v < d) out[bh * d + lane + 64 * v] = (bf16)(acc[v] / ll * gt);
 }
 
-template <int DPAD, bool TERMS>
+template <int DPAD, bool TERMS, bool LOGI = false>
 static int launch_prefill_v(const bf16* q, const bf16* k_new, const bf16* vt_new, int vt_cols,
                           const int* tile_off, const bf16* pages, const int* table, int table_stride, int ring_pages, const int* row_pos,
                           const int* cu_seqlens, const int* n_cached, int B, int n_tiles, int nq, int nkv,
@@ -1051,11 +1082,11 @@ static int launch_prefill_v(const bf16* q, const bf16* k_new, const bf16* vt_new
   if (smem > 48 * 1024) {
     static bool raised = false;
     if (!raised) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_kernel<DPAD, false, TERMS>),
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_kernel<DPAD, false, TERMS, LOGI>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
       if constexpr (can_lean)
         if (e == hipSuccess)
-          e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_kernel<DPAD, true, TERMS>),
+          e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_kernel<DPAD, true, TERMS, LOGI>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
       if (e != hipSuccess) {
         set_error("attn_prefill: cannot have %zu bytes of LDS: %s", smem, hipGetErrorString(e));
@@ -1071,12 +1102,12 @@ static int launch_prefill_v(const bf16* q, const bf16* k_new, const bf16* vt_new
   }
   const unsigned grid = (unsigned)total;
   if (can_lean && d == DPAD)
-    attn_prefill_kernel<DPAD, can_lean, TERMS><<<grid, 256, smem, st>>>(q, k_new, vt_new, vt_cols, tile_off, pages, table,
+    attn_prefill_kernel<DPAD, can_lean, TERMS, LOGI><<<grid, 256, smem, st>>>(q, k_new, vt_new, vt_cols, tile_off, pages, table,
                                                              table_stride, ring_pages, row_pos, cu_seqlens,
                                                              n_cached, B, n_tiles, nq, nkv, d, window, scale, out,
                                                              items, part, part_ways, terms);
   else
-    attn_prefill_kernel<DPAD, false, TERMS><<<grid, 256, smem, st>>>(q, k_new, vt_new, vt_cols, tile_off, pages, table,
+    attn_prefill_kernel<DPAD, false, TERMS, LOGI><<<grid, 256, smem, st>>>(q, k_new, vt_new, vt_cols, tile_off, pages, table,
                                                               table_stride, ring_pages, row_pos, cu_seqlens,
                                                               n_cached, B, n_tiles, nq, nkv, d, window, scale, out,
                                                               items, part, part_ways, terms);
@@ -1098,6 +1129,10 @@ static int launch_prefill(const bf16* q, const bf16* k_new, const bf16* vt_new, 
                           const int* cu_seqlens, const int* n_cached, int B, int n_tiles, int nq, int nkv,
                           int d, int window, float scale, bf16* out, const int4* items, const int4* cut_blocks,
                           int n_cut, float* part, int part_ways, hipStream_t st, const MoreTerms* terms) {
+  if (terms != nullptr && terms->logistic)
+    return launch_prefill_v<DPAD, true, true>(q, k_new, vt_new, vt_cols, tile_off, pages, table, table_stride, ring_pages,
+                                              row_pos, cu_seqlens, n_cached, B, n_tiles, nq, nkv, d, window, scale, out,
+                                              items, cut_blocks, n_cut, part, part_ways, st, *terms);
   if (terms != nullptr)
     return launch_prefill_v<DPAD, true>(q, k_new, vt_new, vt_cols, tile_off, pages, table, table_stride, ring_pages,
                                         row_pos, cu_seqlens, n_cached, B, n_tiles, nq, nkv, d, window, scale, out,
@@ -1111,19 +1146,20 @@ static int launch_prefill(const bf16* q, const bf16* k_new, const bf16* vt_new, 
 static bool decode_through_lds = true;
 constexpr int DR_MAX_PAGES = 2048;      // most pages of a sequence that the kernel through LDS keeps the ids of (8 KB)
 
-template <int DPAD>
-static int launch_decode(const bf16* q, const bf16* pages, const int* table, int table_stride,
-                         int ring_pages, const int* row_pos, int B, int nq, int nkv, int d, int window,
-                         float scale, int n_splits, float* part, bf16* out, hipStream_t st, const MoreTerms* terms) {
+// single-token steps with more terms on the scores; LOGI: logistic weights
+template <int DPAD, bool LOGI>
+static int launch_decode_terms(const bf16* q, const bf16* pages, const int* table, int table_stride,
+                               int ring_pages, const int* row_pos, int B, int nq, int nkv, int d, int window,
+                               float scale, int n_splits, float* part, bf16* out, hipStream_t st, const MoreTerms* terms) {
   const int g = nq / nkv, head_groups = (g + 15) / 16;
   dim3 grid(B * nkv * head_groups, n_splits);
   if constexpr (DPAD == 64 || DPAD == 128 || DPAD == 256) {
-    if (terms != nullptr && d == DPAD && decode_through_lds && table_stride <= DR_MAX_PAGES) {
+    if (d == DPAD && decode_through_lds && table_stride <= DR_MAX_PAGES) {
       constexpr int NS = DPAD == 64 ? 4 : 2;
       constexpr int LDS = NS * PAGE * DPAD * 4 + DR_MAX_PAGES * 4;
       static bool raised_terms = false;
       if (!raised_terms) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_decode_ring_kernel<DPAD, NS, true>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_decode_ring_kernel<DPAD, NS, true, LOGI>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
         if (e != hipSuccess) {
           set_error("attn_decode: cannot have %d bytes of LDS: %s", LDS, hipGetErrorString(e));
@@ -1131,9 +1167,9 @@ static int launch_decode(const bf16* q, const bf16* pages, const int* table, int
         }
         raised_terms = true;
       }
-      attn_decode_ring_kernel<DPAD, NS, true><<<grid, DC_WAVES * 64, LDS, st>>>(q, pages, table, table_stride, ring_pages,
-                                                                                row_pos, nq, nkv, window, scale, n_splits,
-                                                                                head_groups, part, out, *terms);
+      attn_decode_ring_kernel<DPAD, NS, true, LOGI><<<grid, DC_WAVES * 64, LDS, st>>>(q, pages, table, table_stride, ring_pages,
+                                                                                      row_pos, nq, nkv, window, scale, n_splits,
+                                                                                      head_groups, part, out, *terms);
       TL_LAUNCH_CHECK("attn_decode_ring with terms");
       if (n_splits > 1) {
         attn_decode_combine_kernel<<<B * nq, 64, 0, st>>>(part, n_splits, d, out, terms->gate);
@@ -1142,22 +1178,35 @@ static int launch_decode(const bf16* q, const bf16* pages, const int* table, int
       return 0;
     }
   }
-  if (terms != nullptr) {         // more terms on the scores, other head sizes: the kernel that reads the pages into registers
-    if (d == DPAD)
-      attn_decode_kernel<DPAD, true, true><<<grid, DC_WAVES * 64, 0, st>>>(q, pages, table, table_stride, ring_pages,
-                                                                            row_pos, nq, nkv, d, window, scale, n_splits,
-                                                                            head_groups, part, out, *terms);
-    else
-      attn_decode_kernel<DPAD, false, true><<<grid, DC_WAVES * 64, 0, st>>>(q, pages, table, table_stride, ring_pages,
-                                                                             row_pos, nq, nkv, d, window, scale, n_splits,
-                                                                             head_groups, part, out, *terms);
-    TL_LAUNCH_CHECK("attn_decode with terms");
-    if (n_splits > 1) {
-      attn_decode_combine_kernel<<<B * nq, 64, 0, st>>>(part, n_splits, d, out, terms->gate);
-      TL_LAUNCH_CHECK("attn_decode_combine");
-    }
-    return 0;
+  // other head sizes: the kernel that reads the pages into registers
+  if (d == DPAD)
+    attn_decode_kernel<DPAD, true, true, LOGI><<<grid, DC_WAVES * 64, 0, st>>>(q, pages, table, table_stride, ring_pages,
+                                                                                row_pos, nq, nkv, d, window, scale, n_splits,
+                                                                                head_groups, part, out, *terms);
+  else
+    attn_decode_kernel<DPAD, false, true, LOGI><<<grid, DC_WAVES * 64, 0, st>>>(q, pages, table, table_stride, ring_pages,
+                                                                                 row_pos, nq, nkv, d, window, scale, n_splits,
+                                                                                 head_groups, part, out, *terms);
+  TL_LAUNCH_CHECK("attn_decode with terms");
+  if (n_splits > 1) {
+    attn_decode_combine_kernel<<<B * nq, 64, 0, st>>>(part, n_splits, d, out, terms->gate);
+    TL_LAUNCH_CHECK("attn_decode_combine");
   }
+  return 0;
+}
+
+template <int DPAD>
+static int launch_decode(const bf16* q, const bf16* pages, const int* table, int table_stride,
+                         int ring_pages, const int* row_pos, int B, int nq, int nkv, int d, int window,
+                         float scale, int n_splits, float* part, bf16* out, hipStream_t st, const MoreTerms* terms) {
+  const int g = nq / nkv, head_groups = (g + 15) / 16;
+  dim3 grid(B * nkv * head_groups, n_splits);
+  if (terms != nullptr && terms->logistic)
+    return launch_decode_terms<DPAD, true>(q, pages, table, table_stride, ring_pages, row_pos, B, nq, nkv, d, window, scale,
+                                           n_splits, part, out, st, terms);
+  if (terms != nullptr)
+    return launch_decode_terms<DPAD, false>(q, pages, table, table_stride, ring_pages, row_pos, B, nq, nkv, d, window, scale,
+                                            n_splits, part, out, st, terms);
   if constexpr (DPAD == 64 || DPAD == 128 || DPAD == 256) {
     if (d == DPAD && decode_through_lds && table_stride <= DR_MAX_PAGES) {
       constexpr int NS = DPAD == 64 ? 4 : 2;         // 64 KB of LDS, two workgroups a compute unit; heads of 256: 128 KB, one
@@ -1275,11 +1324,14 @@ extern "C" int tl_attn_prefill_terms_bf16(const void* q, const void* k_new, cons
                                           const int* tile_off, const void* pages, const int* table, int table_stride,
                                           int ring_pages, const int* row_pos, const int* cu_seqlens,
                                           const int* n_cached, int B, int n_tiles, int nq, int nkv, int d,
-                                          int window, int keep_first, float scale, const float* slopes,
-                                          const float* sinks, const float* gate, void* out, hipStream_t st) {
+                                          int window, int keep_first, int chunk, float scale, const float* slopes,
+                                          const float* sinks, const float* gate, int logistic, const float* score_bias,
+                                          void* out, hipStream_t st) {
   TL_REQUIRE(keep_first >= 0 && (keep_first == 0 || window == 0 || (long long)ring_pages * PAGE >= (1LL << 24)),
              "attn_prefill: first positions that stay visible beside a window need a cache that keeps every position");
-  const MoreTerms terms{slopes, sinks, gate, window > 0 ? keep_first : 0};
+  TL_REQUIRE(chunk >= 0 && (!logistic || sinks == nullptr) && (logistic || score_bias == nullptr),
+             "attn_prefill: %d positions a chunk; logistic weights have no sink, a softmax no bias on the score", chunk);
+  const MoreTerms terms{slopes, sinks, gate, window > 0 ? keep_first : 0, chunk, logistic, score_bias};
   return attn_prefill_entry(q, k_new, vt_new, vt_cols, tile_off, pages, table, table_stride, ring_pages, row_pos,
                             cu_seqlens, n_cached, B, n_tiles, nq, nkv, d, window, scale, out, nullptr, nullptr, 0,
                             nullptr, 0, 0, 0, st, &terms);
@@ -1321,12 +1373,14 @@ extern "C" int tl_attn_decode_bf16(const void* q, const void* pages, const int* 
 // The same with more terms on the scores (slopes [nq], sinks [nq], gate [B, nq]; each may be null)
 extern "C" int tl_attn_decode_terms_bf16(const void* q, const void* pages, const int* table, int table_stride,
                                          int ring_pages, const int* row_pos, int B, int nq, int nkv, int d,
-                                         int window, int keep_first, float scale, int n_splits, float* part,
-                                         const float* slopes, const float* sinks, const float* gate, void* out,
-                                         hipStream_t st) {
+                                         int window, int keep_first, int chunk, float scale, int n_splits, float* part,
+                                         const float* slopes, const float* sinks, const float* gate, int logistic,
+                                         const float* score_bias, void* out, hipStream_t st) {
   TL_REQUIRE(keep_first >= 0 && (keep_first == 0 || window == 0 || (long long)ring_pages * PAGE >= (1LL << 24)),
              "attn_decode: first positions that stay visible beside a window need a cache that keeps every position");
-  const MoreTerms terms{slopes, sinks, gate, window > 0 ? keep_first : 0};
+  TL_REQUIRE(chunk >= 0 && (!logistic || sinks == nullptr) && (logistic || score_bias == nullptr),
+             "attn_decode: %d positions a chunk; logistic weights have no sink, a softmax no bias on the score", chunk);
+  const MoreTerms terms{slopes, sinks, gate, window > 0 ? keep_first : 0, chunk, logistic, score_bias};
   return attn_decode_entry(q, pages, table, table_stride, ring_pages, row_pos, B, nq, nkv, d, window, scale, n_splits,
                            part, out, st, &terms);
 }

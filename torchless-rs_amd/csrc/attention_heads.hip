@@ -8,6 +8,8 @@
 //     (optional; q and k have a weight each);
 //   * the first `rotary_dim` channels of every head of q and k are rotated in pairs
 //     (i, i + rotary_dim/2) by the angle pos * inv_freq[i];
+//   * or (`unit_norm`) every head of q and of k is divided by its root mean square AFTER the
+//     rotation, with no weight;
 //   * the values are mixed with those that an earlier layer left for the same row:
 //     v <- (1 - lambda) v + lambda v_first  (`mix` 2), or are left for later layers (`mix` 1);
 //     v_first is float, unrounded;
@@ -15,7 +17,8 @@
 //     any other number.
 //
 // k and v go to rows of their own, or (pages != null: one token a sequence) straight into the
-// page of the row's position.  One wave takes one unit of work: a head of q, a head of k, a
+// page of the row's position; a mixer that reads another's keys and values has none of its own
+// (nkv == 0: the row is [q | g]).  One wave takes one unit of work: a head of q, a head of k, a
 // head of v, or 256 gate channels.
 #include "common.hpp"
 
@@ -31,6 +34,7 @@ struct HeadTerms {
   int mix;                 // 0: none; 1: leave v in v_first; 2: mix with v_first
   float lambda;
   float* v_first;          // [n, nkv*dv] float
+  int unit_norm;           // q and k heads divided by their root mean square after the rotation, no weight
 };
 
 template <typename T>
@@ -80,17 +84,25 @@ head_prepare_kernel(const float* __restrict__ proj, const int* __restrict__ row_
       return a;
     };
     const int half = rot.rotary_dim / 2;
-    for (int c = lane; c < dk; c += WAVE) {
-      float a;
-      if (c >= 2 * half) {
-        a = val(c);
-      } else {
-        const int i = c < half ? c : c - half;
-        float sn, cs, ra, rb;
-        sincosf((float)pos * rot.inv_freq[i], &sn, &cs);
-        rotate_pair(val(i), val(i + half), cs, sn, ra, rb);
-        a = c < half ? ra : rb;
+    auto rotated = [&](int c) {
+      if (c >= 2 * half) return val(c);
+      const int i = c < half ? c : c - half;
+      float sn, cs, ra, rb;
+      sincosf((float)pos * rot.inv_freq[i], &sn, &cs);
+      rotate_pair(val(i), val(i + half), cs, sn, ra, rb);
+      return c < half ? ra : rb;
+    };
+    float after = 1.f;
+    if (t.unit_norm) {
+      float ss = 0.f;
+      for (int c = lane; c < dk; c += WAVE) {
+        const float a = rotated(c);
+        ss += a * a;
       }
+      after = 1.0f / sqrtf(wave_sum(ss) / (float)dk + t.eps);
+    }
+    for (int c = lane; c < dk; c += WAVE) {
+      const float a = rotated(c) * after;
       const T o = from_f32<T>(a);
       if (is_q) q[(size_t)n * Q + head * dk + c] = o;
       else if (pages) kd[((size_t)head * PAGE + r) * dk + c] = o;
@@ -123,22 +135,23 @@ using namespace tl;
 extern "C" {
 
 int tl_head_prepare(const float* proj, const int* row_pos, const float* inv_freq, int rotary_dim, const float* bias,
-                    const float* q_norm, const float* k_norm, float eps, int mix, float lambda, float* v_first, int n,
-                    int nq, int nkv, int dk, int dv, int ng, void* q, void* k, void* v, float* gate, int dt,
+                    const float* q_norm, const float* k_norm, float eps, int unit_norm, int mix, float lambda, float* v_first,
+                    int n, int nq, int nkv, int dk, int dv, int ng, void* q, void* k, void* v, float* gate, int dt,
                     const int* table, int table_stride, int ring_pages, void* pages, hipStream_t st) {
-  TL_REQUIRE(n >= 0 && nq > 0 && nkv > 0 && dk > 0 && dv > 0 && ng >= 0 && dk <= HP_MAX_D && dv <= HP_MAX_D,
+  TL_REQUIRE(n >= 0 && nq > 0 && nkv >= 0 && dk > 0 && dv > 0 && ng >= 0 && dk <= HP_MAX_D && dv <= HP_MAX_D,
              "head_prepare: bad sizes n=%d nq=%d nkv=%d dk=%d dv=%d ng=%d (heads up to %d)", n, nq, nkv, dk, dv, ng, HP_MAX_D);
   TL_REQUIRE(rotary_dim >= 0 && rotary_dim % 2 == 0 && rotary_dim <= dk,
              "head_prepare: %d rotated channels of a head of %d (even, at most the head)", rotary_dim, dk);
   TL_REQUIRE(rotary_dim == 0 || inv_freq, "head_prepare: a rotation without frequencies");
-  TL_REQUIRE(proj && row_pos && q && (pages || (k && v)), "head_prepare: a buffer is missing");
+  TL_REQUIRE(proj && row_pos && q && (nkv == 0 || pages || (k && v)), "head_prepare: a buffer is missing");
+  TL_REQUIRE(!unit_norm || (q_norm == nullptr && k_norm == nullptr), "head_prepare: a norm before the rotation or one after it");
   TL_REQUIRE(ng == 0 || gate, "head_prepare: %d gate channels and nowhere to put them", ng);
   TL_REQUIRE(mix >= 0 && mix <= 2 && (mix == 0 || v_first), "head_prepare: mixing values needs the buffer they are left in");
   TL_REQUIRE(pages == nullptr || (table && table_stride > 0 && ring_pages > 0), "head_prepare: pages without a page table");
   TL_REQUIRE(dt == DT_F32 || dt == DT_BF16, "head_prepare: unknown dtype code %d", dt);
   if (n == 0) return 0;
   const Rotation rot{inv_freq, rotary_dim, 0};
-  const HeadTerms t{bias, q_norm, k_norm, eps, mix, lambda, v_first};
+  const HeadTerms t{bias, q_norm, k_norm, eps, mix, lambda, v_first, unit_norm};
   const int units = nq + 2 * nkv + (ng + 255) / 256;
   const dim3 grid(n, (units + 3) / 4);
   if (dt == DT_F32)

@@ -7,6 +7,11 @@
 //   w(p, j) = exp(s(p, j)) / (exp(sink[h]) + sum_j' exp(s(p, j')))
 //   out     = gate[row, h] * sum_j w(p, j) v_j                (sink, gate: optional)
 //
+// With `chunk` C > 0 the key must also lie in the query's run of C positions counted from the
+// sequence's start, floor(j / C) = floor(p / C).  With `logistic` the weights are not a softmax:
+// w(p, j) = 1 / (1 + exp(-(s(p, j) + score_bias[h]))), every key by itself, no normalisation (and
+// no sink).
+//
 // The sink is a score without a key: it takes part in the normalisation once, is
 // neither scaled nor biased, and brings no value.  Scores, weights and the sums over
 // values are float whatever the storage type is.
@@ -31,6 +36,9 @@ struct ScoreTerms {
   const float* slopes;     // [nq] or null
   const float* sinks;      // [nq] or null
   const float* gate;       // [n, nq] or null
+  int chunk;               // 0: none; else a key is seen only inside the query's run of `chunk` positions
+  int logistic;            // the weights are logistic functions of the scores, not a softmax
+  const float* score_bias; // [nq] or null: added to the score (logistic weights only)
 };
 
 // One wave per (row, head): the kernel of the 32-bit path and of every shape that the
@@ -54,7 +62,10 @@ attn_scored_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_new, c
   const int cached = n_cached[b];
   const int row0 = cu_seqlens[b];
   const int window = terms.window;
-  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  if (terms.chunk > 0) lo = max(lo, (p / terms.chunk) * terms.chunk);
+  const float sbias = terms.score_bias ? terms.score_bias[h] : 0.f;
+  const bool logistic = terms.logistic != 0;
   const size_t keys_elems = (size_t)nkv * PAGE * dk;
   const size_t page_elems = (size_t)nkv * PAGE * (dk + dv);
   const float slope = terms.slopes ? terms.slopes[h] : 0.f;
@@ -95,13 +106,19 @@ attn_scored_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_new, c
       }
       float dot = 0.f;
       for (int t = 0; t < dk; ++t) dot = fmaf(to_f32(kp[t]), q_s[t], dot);
-      s = dot * terms.scale - slope * (float)(p - j);
+      s = dot * terms.scale - slope * (float)(p - j) + sbias;
     }
-    const float m_new = fmaxf(m, wave_max(s));       // finite: key j0 is visible
-    const float pj = (j < end) ? expf(s - m_new) : 0.f;
-    const float alpha = expf(m - m_new);              // 0 in the first tile without a sink (m = -inf)
-    l = l * alpha + wave_sum(pj);
-    m = m_new;
+    float pj, alpha;
+    if (logistic) {                                   // every key by itself: no maximum, no sum
+      pj = (j < end) ? 1.0f / (1.0f + expf(-s)) : 0.f;
+      alpha = 1.f;
+    } else {
+      const float m_new = fmaxf(m, wave_max(s));     // finite: key j0 is visible
+      pj = (j < end) ? expf(s - m_new) : 0.f;
+      alpha = expf(m - m_new);                        // 0 in the first tile without a sink (m = -inf)
+      l = l * alpha + wave_sum(pj);
+      m = m_new;
+    }
     __syncthreads();
     p_s[lane] = pj;
     v_s[lane] = vp;
@@ -124,7 +141,7 @@ attn_scored_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_new, c
 #pragma unroll
   for (int i = 0; i < SC_MAX_D / WAVE; ++i) {
     const int dim = lane + WAVE * i;
-    if (dim < dv) o[dim] = from_f32<TO>((acc[i] / l) * g);
+    if (dim < dv) o[dim] = from_f32<TO>((logistic ? acc[i] : acc[i] / l) * g);
   }
 }
 
@@ -348,8 +365,11 @@ extern "C" {
 int tl_attn_scored_plain(const void* q, const void* k_new, const void* v_new, const void* pages, int dt,
                          const int* table, int table_stride, int ring_pages, const int* row_seq,
                          const int* row_pos, const int* cu_seqlens, const int* n_cached, int n, int nq,
-                         int nkv, int dk, int dv, int window, int keep_first, float scale, const float* slopes,
-                         const float* sinks, const float* gate, void* out, int out_dt, hipStream_t st) {
+                         int nkv, int dk, int dv, int window, int keep_first, int chunk, float scale, const float* slopes,
+                         const float* sinks, const float* gate, int logistic, const float* score_bias, void* out, int out_dt,
+                         hipStream_t st) {
+  TL_REQUIRE(chunk >= 0 && (!logistic || sinks == nullptr) && (logistic || score_bias == nullptr),
+             "scored attention: %d positions a chunk; logistic weights have no sink, a softmax no bias on the score", chunk);
   TL_REQUIRE(out_dt == dt || out_dt == DT_F32, "scored attention: the result is of the operands' type or float");
   TL_REQUIRE(n >= 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "scored attention: bad head counts nq=%d nkv=%d",
              nq, nkv);
@@ -362,7 +382,7 @@ int tl_attn_scored_plain(const void* q, const void* k_new, const void* v_new, co
              "scored attention: first positions that stay visible beside a window need a cache that keeps every position");
   TL_REQUIRE((long long)n * nq < 2147483647LL, "scored attention: too many (row, head) pairs");
   if (n == 0) return 0;
-  const ScoreTerms terms{scale, window, window > 0 ? keep_first : 0, slopes, sinks, gate};
+  const ScoreTerms terms{scale, window, window > 0 ? keep_first : 0, slopes, sinks, gate, chunk, logistic, score_bias};
   if (dt == DT_F32)
     attn_scored_plain_kernel<float, float><<<n * nq, 64, 0, st>>>(
         (const float*)q, (const float*)k_new, (const float*)v_new, (const float*)pages, table, table_stride,

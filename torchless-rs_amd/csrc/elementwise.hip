@@ -483,7 +483,7 @@ __global__ void silu_mul_pairs_kernel(const bf16* __restrict__ gu, long long chu
   *reinterpret_cast<bf16x8*>(out + n * I + group * 32 + part * 8) = o;
 }
 
-// ---- layer norm with a weight and no bias: y = (x - mean) / sqrt(var + eps) * w -------------
+// ---- layer norm with a weight and an optional bias: y = (x - mean) / sqrt(var + eps) * w + beta ----
 // var is the mean of the squared deviations from the mean (two passes over the row, both in
 // float).  The row may get a bias first (z + b, the bias of the product that made z).
 // `x` null: y is written to `out`.  `x` given: the norm is ADDED to the stream, x += y, and
@@ -492,7 +492,7 @@ __global__ void silu_mul_pairs_kernel(const bf16* __restrict__ gu, long long chu
 template <typename TO>
 __global__ void __launch_bounds__(256)
 layernorm_kernel(const float* __restrict__ z, const float* __restrict__ bias, const float* __restrict__ w,
-                 float eps, float* __restrict__ x, TO* __restrict__ out, int H) {
+                 const float* __restrict__ beta, float eps, float* __restrict__ x, TO* __restrict__ out, int H) {
   __shared__ float sh[4];
   const int n = blockIdx.x;
   const float* zr = z + (size_t)n * H;
@@ -506,7 +506,7 @@ layernorm_kernel(const float* __restrict__ z, const float* __restrict__ bias, co
   }
   const float sd = sqrtf(block_sum<256>(ss, sh) / (float)H + eps);
   for (int i = threadIdx.x; i < H; i += 256) {
-    const float y = ((zr[i] + (bias ? bias[i] : 0.f) - mean) / sd) * w[i];
+    const float y = ((zr[i] + (bias ? bias[i] : 0.f) - mean) / sd) * w[i] + (beta ? beta[i] : 0.f);
     if (x) {
       const float xn = x[(size_t)n * H + i] + y;
       x[(size_t)n * H + i] = xn;
@@ -521,7 +521,7 @@ layernorm_kernel(const float* __restrict__ z, const float* __restrict__ bias, co
 template <typename TO, int IT>
 __global__ void __launch_bounds__(256)
 layernorm_reg_kernel(const float* __restrict__ z, const float* __restrict__ bias, const float* __restrict__ w,
-                     float eps, float* __restrict__ x, TO* __restrict__ out, int H) {
+                     const float* __restrict__ beta, float eps, float* __restrict__ x, TO* __restrict__ out, int H) {
   __shared__ float sh[4];
   const int n = blockIdx.x;
   const float4* zr = reinterpret_cast<const float4*>(z + (size_t)n * H);
@@ -560,6 +560,10 @@ layernorm_reg_kernel(const float* __restrict__ z, const float* __restrict__ bias
       const float4 g = wr[c];
       float4 y;
       y.x = (v[i].x / sd) * g.x; y.y = (v[i].y / sd) * g.y; y.z = (v[i].z / sd) * g.z; y.w = (v[i].w / sd) * g.w;
+      if (beta) {
+        const float4 e = reinterpret_cast<const float4*>(beta)[c];
+        y.x += e.x; y.y += e.y; y.z += e.z; y.w += e.w;
+      }
       if (x) {
         float4* xr = reinterpret_cast<float4*>(x + (size_t)n * H);
         float4 a = xr[c];
@@ -993,26 +997,27 @@ int tl_silu_mul_pairs(const void* gu, int n, int I, void* out, hipStream_t st) {
 }
 
 // x null: out = layernorm(z + bias); else x += layernorm(z + bias) and out (may be null) = x
-int tl_layernorm(const float* z, const float* bias, const float* w, float eps, float* x, void* out, int out_dt,
-                 int n, int H, hipStream_t st) {
+int tl_layernorm(const float* z, const float* bias, const float* w, const float* beta, float eps, float* x, void* out,
+                 int out_dt, int n, int H, hipStream_t st) {
   TL_REQUIRE(n >= 0 && H > 0, "layernorm: bad sizes n=%d H=%d", n, H);
   TL_REQUIRE(x != nullptr || out != nullptr, "layernorm: nowhere to write");
   TL_REQUIRE(out == nullptr || out_dt == DT_F32 || out_dt == DT_BF16, "layernorm: unknown dtype code %d", out_dt);
   if (n == 0) return 0;
-  const bool al = (uintptr_t)z % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)bias % 16 == 0 && (uintptr_t)x % 16 == 0;
+  const bool al = (uintptr_t)z % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)bias % 16 == 0 && (uintptr_t)x % 16 == 0 &&
+                  (uintptr_t)beta % 16 == 0;
   const bool vec = H % 4 == 0 && H <= 8192 && al;
   const bool f32 = out == nullptr || out_dt == DT_F32;
-#define TL_LN(IT)                                                                                        \
-  do {                                                                                                   \
-    if (f32) layernorm_reg_kernel<float, IT><<<n, 256, 0, st>>>(z, bias, w, eps, x, (float*)out, H);     \
-    else layernorm_reg_kernel<bf16, IT><<<n, 256, 0, st>>>(z, bias, w, eps, x, (bf16*)out, H);           \
+#define TL_LN(IT)                                                                                              \
+  do {                                                                                                         \
+    if (f32) layernorm_reg_kernel<float, IT><<<n, 256, 0, st>>>(z, bias, w, beta, eps, x, (float*)out, H);     \
+    else layernorm_reg_kernel<bf16, IT><<<n, 256, 0, st>>>(z, bias, w, beta, eps, x, (bf16*)out, H);           \
   } while (0)
   if (vec && H <= 1024) TL_LN(1);
   else if (vec && H <= 2048) TL_LN(2);
   else if (vec && H <= 4096) TL_LN(4);
   else if (vec) TL_LN(8);
-  else if (f32) layernorm_kernel<float><<<n, 256, 0, st>>>(z, bias, w, eps, x, (float*)out, H);
-  else layernorm_kernel<bf16><<<n, 256, 0, st>>>(z, bias, w, eps, x, (bf16*)out, H);
+  else if (f32) layernorm_kernel<float><<<n, 256, 0, st>>>(z, bias, w, beta, eps, x, (float*)out, H);
+  else layernorm_kernel<bf16><<<n, 256, 0, st>>>(z, bias, w, beta, eps, x, (bf16*)out, H);
 #undef TL_LN
   TL_LAUNCH_CHECK("layernorm");
   return 0;

@@ -1,6 +1,7 @@
 // A routed mixture of small feed-forward layers ("experts").
 //
-// Router, per row, in float: z = W_r h, s = softmax(z) over all E experts.  The experts form
+// Router, per row, in float: z = W_r h, s = softmax(z) over all E experts (or, `logistic`, every
+// expert's own 1 / (1 + exp(-z))).  The experts form
 // `groups` equal groups of neighbours; a group's score is its largest s, and only experts of the
 // `keep` best groups can be chosen (groups == 0: every expert can).  Of those the `top` with the
 // largest s are chosen; their weights are their s, not renormalised.  Of equal scores the one
@@ -20,7 +21,7 @@ constexpr int RT_MAX_E = 1024;
 template <typename T>
 __global__ void __launch_bounds__(256)
 route_kernel(const T* __restrict__ h, int W, const float* __restrict__ wr, int E, int groups, int keep, int top,
-             float* __restrict__ weights, int* __restrict__ chosen, bool vec) {
+             int logistic, float* __restrict__ weights, int* __restrict__ chosen, bool vec) {
   __shared__ float s_s[RT_MAX_E];
   __shared__ float g_s[RT_MAX_E];
   __shared__ unsigned char ok_s[RT_MAX_E];
@@ -56,14 +57,18 @@ route_kernel(const T* __restrict__ h, int W, const float* __restrict__ wr, int E
     if (lane == 0) s_s[e] = dot;
   }
   __syncthreads();
-  float m = -INFINITY;
-  for (int e = t; e < E; e += 256) m = fmaxf(m, s_s[e]);
-  m = block_max<256>(m, sh);
-  float sum = 0.f;
-  for (int e = t; e < E; e += 256) sum += expf(s_s[e] - m);
-  sum = block_sum<256>(sum, sh);
-  __syncthreads();
-  for (int e = t; e < E; e += 256) s_s[e] = expf(s_s[e] - m) / sum;
+  if (logistic) {                                      // every expert's score by itself
+    for (int e = t; e < E; e += 256) s_s[e] = 1.0f / (1.0f + expf(-s_s[e]));
+  } else {
+    float m = -INFINITY;
+    for (int e = t; e < E; e += 256) m = fmaxf(m, s_s[e]);
+    m = block_max<256>(m, sh);
+    float sum = 0.f;
+    for (int e = t; e < E; e += 256) sum += expf(s_s[e] - m);
+    sum = block_sum<256>(sum, sh);
+    __syncthreads();
+    for (int e = t; e < E; e += 256) s_s[e] = expf(s_s[e] - m) / sum;
+  }
   __syncthreads();
   if (groups > 0) {
     const int per = E / groups;
@@ -207,14 +212,94 @@ expert_rows_down_kernel(const T* __restrict__ hs, const T* __restrict__ down, co
   }
 }
 
+
+// ---- gated experts ----------------------------------------------------------------------------------------
+// An expert with a gate: down(act(g, u)) with g = W_gate t, u = W_up t and
+//     act(g, u) = g' logistic(alpha g') (u' + shift) ,  g' = min(g, limit) ,  u' = clamp(u, -limit, limit).
+// The stacked matrix holds, expert after expert, the rows [gate (ff) | up (ff)], and behind the last expert
+// the shared one's [gate (shared) | up (shared)], which has a limit of its own.  The router's weight s
+// multiplies the expert's INPUT t = s y (`on_input`: g and u are linear in t, so s multiplies both before
+// the clamps) or its output (the activation times s).  An expert with weight 0 adds nothing either way.
+struct GateTerms {
+  float limit, limit_shared, alpha, shift;
+  int on_input;
+};
+
+__device__ __forceinline__ float gated_value(float g, float u, float s, float limit, const GateTerms& k) {
+  if (k.on_input) {
+    g *= s;
+    u *= s;
+  }
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  const float a = g / (1.0f + expf(-k.alpha * g)) * (u + k.shift);
+  return k.on_input ? a : a * s;
+}
+
+// out[n, j] for the E * ff + shared hidden channels j; gu float [n, 2 (E * ff + shared)] as the stacked matrix
+// lays it; weights [n, E] (E == 0: none; a column of weight 1 for the shared part)
+template <typename T>
+__global__ void __launch_bounds__(256)
+expert_gated_act_kernel(const float* __restrict__ gu, const float* __restrict__ weights, int E, int ff, int shared,
+                        GateTerms k, T* __restrict__ out) {
+  const int n = blockIdx.x;
+  const int total = E * ff + shared;
+  const float* row = gu + (size_t)n * 2 * total;
+  for (int j = blockIdx.y * 256 + threadIdx.x; j < total; j += gridDim.y * 256) {
+    float a;
+    if (j < E * ff) {
+      const int e = j / ff, c = j % ff;
+      a = gated_value(row[2 * e * ff + c], row[2 * e * ff + ff + c], weights[(size_t)n * E + e], k.limit, k);
+    } else {
+      const int c = j - E * ff;
+      a = gated_value(row[2 * E * ff + c], row[2 * E * ff + shared + c], 1.f, k.limit_shared, k);
+    }
+    out[(size_t)n * total + j] = from_f32<T>(a);
+  }
+}
+
+// the chosen experts alone: hs[n, k * ff + j] = act of expert chosen[n, k]'s rows j against y[n], and the shared
+// expert's behind them; `up` is the stacked matrix [2 (E * ff + shared), H]
+template <typename T>
+__global__ void __launch_bounds__(256)
+expert_rows_gated_up_kernel(const T* __restrict__ y, int H, const T* __restrict__ up, const int* __restrict__ chosen,
+                            const float* __restrict__ weights, int E, int top, int ff, int shared, GateTerms kt, bool vec,
+                            T* __restrict__ hs) {
+  const int slots = top + (shared ? 1 : 0);
+  const int n = blockIdx.x / slots, k = blockIdx.x % slots;
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  int base, count;
+  float scale = 1.f, limit = kt.limit_shared;
+  if (k < top) {
+    const int e = chosen[(size_t)n * top + k];
+    base = 2 * e * ff;
+    count = ff;
+    scale = weights[(size_t)n * E + e];
+    limit = kt.limit;
+  } else {
+    base = 2 * E * ff;
+    count = shared;
+  }
+  const T* row = y + (size_t)n * H;
+  T* out = hs + (size_t)n * (top * ff + shared) + (size_t)k * ff;
+#pragma unroll
+  for (int r = 0; r < ER_ROWS / 4; ++r) {
+    const int j = blockIdx.y * ER_ROWS + wave * (ER_ROWS / 4) + r;
+    if (j >= count) break;
+    const float g = wave_dot(up + (size_t)(base + j) * H, row, H, vec, lane);
+    const float u = wave_dot(up + (size_t)(base + count + j) * H, row, H, vec, lane);
+    if (lane == 0) out[j] = from_f32<T>(gated_value(g, u, scale, limit, kt));
+  }
+}
+
 }  // namespace tl
 
 using namespace tl;
 
 extern "C" {
 
-int tl_route(const void* h, int dt, int n, int W, const float* wr, int E, int groups, int keep, int top, float* weights,
-             int* chosen, hipStream_t st) {
+int tl_route(const void* h, int dt, int n, int W, const float* wr, int E, int groups, int keep, int top, int logistic,
+             float* weights, int* chosen, hipStream_t st) {
   TL_REQUIRE(n >= 0 && W > 0 && E > 0 && E <= RT_MAX_E && top > 0 && top <= E, "route: bad sizes n=%d W=%d E=%d top=%d (experts up to %d)",
              n, W, E, top, RT_MAX_E);
   TL_REQUIRE(groups >= 0 && (groups == 0 || (E % groups == 0 && keep > 0 && keep <= groups && keep * (E / groups) >= top)),
@@ -223,9 +308,9 @@ int tl_route(const void* h, int dt, int n, int W, const float* wr, int E, int gr
   if (n == 0) return 0;
   const bool vec = W % 4 == 0 && (uintptr_t)h % 16 == 0 && (uintptr_t)wr % 16 == 0;
   if (dt == DT_F32)
-    route_kernel<float><<<n, 256, 0, st>>>((const float*)h, W, wr, E, groups, keep, top, weights, chosen, vec);
+    route_kernel<float><<<n, 256, 0, st>>>((const float*)h, W, wr, E, groups, keep, top, logistic, weights, chosen, vec);
   else if (dt == DT_BF16)
-    route_kernel<bf16><<<n, 256, 0, st>>>((const bf16*)h, W, wr, E, groups, keep, top, weights, chosen, vec);
+    route_kernel<bf16><<<n, 256, 0, st>>>((const bf16*)h, W, wr, E, groups, keep, top, logistic, weights, chosen, vec);
   else
     TL_REQUIRE(false, "route: unknown dtype code %d", dt);
   TL_LAUNCH_CHECK("route");
@@ -288,6 +373,47 @@ int tl_expert_rows_down(const void* hs, const void* down, const int* chosen, int
   else
     expert_rows_down_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)hs, (const bf16*)down, chosen, E, top, ff, shared, H, vec, accumulate, out);
   TL_LAUNCH_CHECK("expert_rows_down");
+  return 0;
+}
+
+// gu float [n, 2 (E * ff + shared)], weights float [n, E] (E == 0: none) -> out [n, E * ff + shared] of dtype dt
+int tl_expert_gated_act(const float* gu, const float* weights, int n, int E, int ff, int shared, float limit, float limit_shared,
+                        float alpha, float shift, int on_input, void* out, int dt, hipStream_t st) {
+  TL_REQUIRE(n >= 0 && E >= 0 && ff >= 0 && shared >= 0 && E * ff + shared > 0, "expert_gated_act: bad sizes E=%d ff=%d shared=%d", E, ff, shared);
+  TL_REQUIRE(gu && out && (E == 0 || weights), "expert_gated_act: a buffer is missing");
+  TL_REQUIRE(dt == DT_F32 || dt == DT_BF16, "expert_gated_act: unknown dtype code %d", dt);
+  if (n == 0) return 0;
+  const int total = E * ff + shared;
+  const dim3 grid(n, min((total + 255) / 256, 64));
+  const GateTerms k{limit, limit_shared, alpha, shift, on_input};
+  if (dt == DT_F32) expert_gated_act_kernel<float><<<grid, 256, 0, st>>>(gu, weights, E, ff, shared, k, (float*)out);
+  else expert_gated_act_kernel<bf16><<<grid, 256, 0, st>>>(gu, weights, E, ff, shared, k, (bf16*)out);
+  TL_LAUNCH_CHECK("expert_gated_act");
+  return 0;
+}
+
+// y [n, H], up [2 (E * ff + shared), H], chosen int [n, top], weights [n, E] -> hs [n, top * ff + shared], all of dtype dt
+int tl_expert_rows_gated_up(const void* y, int H, const void* up, const int* chosen, const float* weights, int n, int E, int top,
+                            int ff, int shared, float limit, float limit_shared, float alpha, float shift, int on_input, void* hs,
+                            int dt, hipStream_t st) {
+  TL_REQUIRE(n >= 0 && H > 0 && E > 0 && top > 0 && top <= E && ff > 0 && shared >= 0,
+             "expert_rows_gated_up: bad sizes H=%d E=%d top=%d ff=%d shared=%d", H, E, top, ff, shared);
+  TL_REQUIRE(y && up && chosen && weights && hs, "expert_rows_gated_up: a buffer is missing");
+  TL_REQUIRE(dt == DT_F32 || dt == DT_BF16, "expert_rows_gated_up: unknown dtype code %d", dt);
+  if (n == 0) return 0;
+  const int slots = top + (shared ? 1 : 0);
+  const int most = ff > shared ? ff : shared;
+  const dim3 grid(n * slots, (most + ER_ROWS - 1) / ER_ROWS);
+  const int per = dt == DT_BF16 ? 8 : 4;
+  const bool vec = H % per == 0 && (uintptr_t)y % 16 == 0 && (uintptr_t)up % 16 == 0;
+  const GateTerms k{limit, limit_shared, alpha, shift, on_input};
+  if (dt == DT_F32)
+    expert_rows_gated_up_kernel<float><<<grid, 256, 0, st>>>((const float*)y, H, (const float*)up, chosen, weights, E, top, ff, shared, k,
+                                                             vec, (float*)hs);
+  else
+    expert_rows_gated_up_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)y, H, (const bf16*)up, chosen, weights, E, top, ff, shared, k,
+                                                            vec, (bf16*)hs);
+  TL_LAUNCH_CHECK("expert_rows_gated_up");
   return 0;
 }
 

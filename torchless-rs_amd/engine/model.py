@@ -42,6 +42,8 @@ class Model:
             if run.kv_from is not None and not (0 <= run.kv_from < i):
                 raise ValueError(f"schedule entry {i} reads the cache of entry {run.kv_from}, which "
                                  "is not an earlier one")
+        if spec.exit is not None and not (0 <= spec.exit[0] < len(self.stream_parts)):
+            raise ValueError(f"the stream part after the last run is number {spec.exit[0]}, there are {len(self.stream_parts)}")
         self.loaded = False
         self.graph_safe = all(p.graph_safe for p in self._all_parts())
 
@@ -160,6 +162,9 @@ class Model:
         for commit in ctx.host.pop("deferred", []):
             commit()
         flush_pending(ctx, x)
+        if self.spec.exit is not None:
+            part, t = self.spec.exit
+            self.stream_parts[part].forward(ctx, x, embedded, t)
         logits = ws.get("logits", (n_want, V), torch.float32)
         if n_want:
             xs = ws.get("head_x", (n_want, H), torch.float32)

@@ -347,9 +347,10 @@ def silu_mul_pairs(gu: torch.Tensor, out: torch.Tensor, activation: str = "silu"
 
 
 def layernorm(z: torch.Tensor, w: torch.Tensor, eps: float, out: Optional[torch.Tensor] = None,
-              add_to: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None) -> None:
-    """Layer norm with a weight and no bias of its own, y = (z - mean) / sqrt(var + eps) * w over
-    z float32 [n, H] (`bias`: added to z first, the bias of the product that made z).  Without
+              add_to: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
+              beta: Optional[torch.Tensor] = None) -> None:
+    """Layer norm, y = (z - mean) / sqrt(var + eps) * w + beta over z float32 [n, H] (`beta`: the norm's
+    own bias, or None; `bias`: added to z first, the bias of the product that made z).  Without
     `add_to`, y goes to `out` (float32 or the compute dtype).  With it, the stream add_to += y,
     and `out`, if given, receives the new stream in its dtype."""
     n, H = z.shape
@@ -357,14 +358,89 @@ def layernorm(z: torch.Tensor, w: torch.Tensor, eps: float, out: Optional[torch.
     _req(w, "layernorm.w", torch.float32, (H,))
     if bias is not None:
         _req(bias, "layernorm.bias", torch.float32, (H,))
+    if beta is not None:
+        _req(beta, "layernorm.beta", torch.float32, (H,))
     if add_to is not None:
         _req(add_to, "layernorm.add_to", torch.float32, (n, H))
     elif out is None:
         raise KernelError("layernorm: needs `out` or `add_to`")
     if out is not None:
         _req(out, "layernorm.out", None, (n, H))
-    _check(lib().tl_layernorm(_p(z), _p(bias), _p(w), ctypes.c_float(eps), _p(add_to), _p(out),
+    _check(lib().tl_layernorm(_p(z), _p(bias), _p(w), _p(beta), ctypes.c_float(eps), _p(add_to), _p(out),
                               _code(out.dtype) if out is not None else DT_F32, n, H, _stream()))
+
+
+def layernorm_rows_in_registers(H: int) -> bool:
+    """Does `layernorm_add_norm` take rows of H channels?"""
+    return H % 4 == 0 and H <= 8192
+
+
+def layernorm_add_norm(z: torch.Tensor, w: torch.Tensor, beta, eps: float, x: torch.Tensor, bias=None,
+                       w_next=None, beta_next=None, eps_next: float = 0.0, out=None) -> None:
+    """x += LN(z + bias; w, beta) and, with `w_next`, out = LN(x; w_next, beta_next) of the new row, in one
+    kernel that holds the row in registers (`layernorm_rows_in_registers`).  z, x float32 [n, H]; out
+    [n, H] float32 or the compute dtype."""
+    n, H = z.shape
+    _req(z, "layernorm_add_norm.z", torch.float32)
+    _req(x, "layernorm_add_norm.x", torch.float32, (n, H))
+    for t, name in ((w, "w"), (beta, "beta"), (bias, "bias"), (w_next, "w_next"), (beta_next, "beta_next")):
+        if t is not None:
+            _req(t, "layernorm_add_norm." + name, torch.float32, (H,))
+    if w_next is not None:
+        _req(out, "layernorm_add_norm.out", None, (n, H))
+    _check(lib().tl_layernorm_add_norm(_p(z), _p(bias), _p(w), _p(beta), ctypes.c_float(eps), _p(x), _p(w_next),
+                                       _p(beta_next) if w_next is not None else None, ctypes.c_float(eps_next),
+                                       _p(out) if w_next is not None else None,
+                                       _code(out.dtype) if w_next is not None else DT_F32, n, H, _stream()))
+
+
+def depth_average(x: torch.Tensor, kept: torch.Tensor, coef: torch.Tensor, t: int) -> None:
+    """kept[t] = x, then x = sum over j <= t of coef[j] * kept[j]: the stream that goes on is a weighted sum
+    of the stream's earlier versions and this one.  x float32 [n, H], kept float32 [>= t + 1, n, H], coef
+    float32 [>= t + 1]."""
+    _req(x, "depth_average.x", torch.float32)
+    _req(kept, "depth_average.kept", torch.float32)
+    _req(coef, "depth_average.coef", torch.float32)
+    if kept.dim() != 3 or tuple(kept.shape[1:]) != tuple(x.shape) or kept.shape[0] <= t or coef.numel() <= t or t < 0:
+        raise KernelError(f"depth_average: version {t} of a stream {tuple(x.shape)} in {tuple(kept.shape)} with "
+                          f"{coef.numel()} weights")
+    _check(lib().tl_depth_average(_p(x), _p(kept), _p(coef), int(t), ctypes.c_longlong(x.numel()), _stream()))
+
+
+def gated_recurrence_chunk() -> int:
+    """Rows in a run of `gated_recurrence`'s second way."""
+    return int(lib().tl_gated_recurrence_chunk())
+
+
+def gated_recurrence(proj: torch.Tensor, bz, bx, state: torch.Tensor, cu_seqlens, slots, out: torch.Tensor,
+                     n_runs: int = 0, scratch=None) -> None:
+    """A gated recurrence per channel over the rows of a step, sequence by sequence.  proj float32 [n, 3 W] =
+    [a | b | g]: z = logistic(a + bz), c = cand(b + bx) (u + 1/2 for u >= 0, logistic(u) below),
+    S <- (1 - z) S + z c, out = S * silu(g).  `state` float32 [slots, >= W] (rows may be strided) is read and
+    left updated.  `n_runs` 0: a thread a (sequence, channel) goes through the rows in order; else the step's
+    number of runs of `gated_recurrence_chunk()` rows (sum over sequences of the rounded-up quotient): a
+    workgroup a run, with `scratch` float32 [>= (2 n_runs + B) W]."""
+    n, W3 = proj.shape
+    W = W3 // 3
+    B = slots.shape[0]
+    _req(proj, "gated_recurrence.proj", torch.float32)
+    if W3 != 3 * W:
+        raise KernelError(f"gated_recurrence: a row of {W3} is not [a | b | g]")
+    for t, name in ((bz, "bz"), (bx, "bx")):
+        if t is not None:
+            _req(t, "gated_recurrence." + name, torch.float32, (W,))
+    if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or not state.is_cuda or state.shape[1] < W:
+        raise KernelError("gated_recurrence.state: float32 [slots, >= W] on the GPU, rows may be strided")
+    _req(cu_seqlens, "gated_recurrence.cu_seqlens", torch.int32, (B + 1,))
+    _req(slots, "gated_recurrence.slots", torch.int32)
+    _req(out, "gated_recurrence.out", None, (n, W))
+    if n_runs:
+        _req(scratch, "gated_recurrence.scratch", torch.float32)
+        if scratch.numel() < (2 * n_runs + B) * W:
+            raise KernelError(f"gated_recurrence: scratch of {scratch.numel()} for {n_runs} runs of {B} sequences")
+    _check(lib().tl_gated_recurrence(_p(proj), _p(bz), _p(bx), n, W, _p(state), ctypes.c_longlong(state.stride(0)),
+                                     _p(cu_seqlens), _p(slots), B, int(n_runs), _p(scratch) if n_runs else None,
+                                     _p(out), _code(out.dtype), _stream()))
 
 
 def cast_rows(x: torch.Tensor, out: torch.Tensor) -> None:
@@ -406,12 +482,31 @@ class ScoreTerms:
     -slope[h] * (p - j) by the distance of query and key; `sinks` (float32 [nq] or None), a score
     per head with no key and no value that takes part in the softmax's sum once; `window`;
     `keep_first`: with a window, the first positions of a sequence that stay visible beside it
-    (the cache must then keep every position: a ring would overwrite them)."""
+    (the cache must then keep every position: a ring would overwrite them); `chunk`: a key is seen
+    only inside the query's run of that many positions counted from the sequence's start,
+    floor(j / chunk) == floor(p / chunk); `logistic`: the weight of a key is
+    1 / (1 + exp(-(score + score_bias[h]))), every key by itself, instead of a softmax over the keys
+    (`score_bias` float32 [nq] or None; no sink)."""
 
     def __init__(self, scale: float, window: Optional[int] = None, slopes: Optional[torch.Tensor] = None,
-                 sinks: Optional[torch.Tensor] = None, keep_first: int = 0):
+                 sinks: Optional[torch.Tensor] = None, keep_first: int = 0, chunk: Optional[int] = None,
+                 logistic: bool = False, score_bias: Optional[torch.Tensor] = None):
         self.scale, self.window, self.slopes, self.sinks = float(scale), (int(window) if window else None), slopes, sinks
         self.keep_first = int(keep_first) if self.window else 0
+        self.chunk = int(chunk) if chunk else 0
+        self.logistic, self.score_bias = bool(logistic), score_bias
+        if self.logistic and sinks is not None:
+            raise KernelError("attention: logistic weights have no sink")
+        if score_bias is not None and not self.logistic:
+            raise KernelError("attention: a bias on the score goes with logistic weights (a softmax does not see it)")
+
+    @property
+    def reach(self) -> Optional[int]:
+        """How many positions back a query may look (None: to the first)."""
+        if self.window and self.keep_first:
+            return None
+        both = [v for v in (self.window, self.chunk) if v]
+        return min(both) if both else None
 
 
 def _req_pages(pages: torch.Tensor, nkv: int, dk: int, dv: int, what: str) -> None:
@@ -447,13 +542,16 @@ def attn_scored_plain(q, k_new, v_new, pages, nkv: int, dv: int, table, ring_pag
         _req(terms.sinks, "attn_scored.sinks", torch.float32, (nq,))
     if gate is not None:
         _req(gate, "attn_scored.gate", torch.float32, (n, nq))
+    if terms.score_bias is not None:
+        _req(terms.score_bias, "attn_scored.score_bias", torch.float32, (nq,))
     if table.dim() != 2 or table.shape[0] != B:
         raise KernelError("attn_scored.table: needs one row per sequence")
     _check(lib().tl_attn_scored_plain(_p(q), _p(k_new), _p(v_new), _p(pages), _code(q.dtype), _p(table),
                                       table.shape[1], ring_pages, _p(row_seq), _p(row_pos), _p(cu_seqlens),
                                       _p(n_cached), n, nq, nkv, dk, dv, int(terms.window or 0), terms.keep_first,
-                                      ctypes.c_float(terms.scale), _p(terms.slopes), _p(terms.sinks), _p(gate),
-                                      _p(out), _code(out.dtype), _stream()))
+                                      terms.chunk, ctypes.c_float(terms.scale), _p(terms.slopes), _p(terms.sinks),
+                                      _p(gate), int(terms.logistic), _p(terms.score_bias), _p(out), _code(out.dtype),
+                                      _stream()))
 
 
 def scored_on_matrix_cores(dtype: torch.dtype, dk: int, dv: int) -> bool:
@@ -469,6 +567,8 @@ def _terms_args(terms: ScoreTerms, gate, n: int, nq: int):
         _req(terms.sinks, "attn_scored.sinks", torch.float32, (nq,))
     if gate is not None:
         _req(gate, "attn_scored.gate", torch.float32, (n, nq))
+    if terms.score_bias is not None:
+        _req(terms.score_bias, "attn_scored.score_bias", torch.float32, (nq,))
     return _p(terms.slopes), _p(terms.sinks), _p(gate)
 
 
@@ -485,14 +585,16 @@ def attention_scored(q, k_new, v_new, pages, nkv: int, dv: int, table, ring_page
         most_pages = table.shape[1]
         if terms.window:          # (kept first positions: the table holds every page, a row reads the window's and the kept ones)
             most_pages = min(most_pages, -(-terms.window // PAGE) + 1 + -(-int(terms.keep_first or 0) // PAGE))
+        if terms.chunk:
+            most_pages = min(most_pages, -(-terms.chunk // PAGE) + 1)
         splits = decode_splits(n, nq, nkv, most_pages, compute_units(q.device), dk)
         part = ctx.workspace.get("attn_part", (n * nq * splits * (dk + 2),), torch.float32)
         _decode_args(q, pages, table, ctx.row_pos, part, out, splits)
         slopes, sinks, gt = _terms_args(terms, gate, n, nq)
         _check(lib().tl_attn_decode_terms_bf16(_p(q), _p(pages), _p(table), table.shape[1], ring_pages, _p(ctx.row_pos),
                                                n, nq, nkv, dk, int(terms.window or 0), int(terms.keep_first or 0),
-                                               ctypes.c_float(terms.scale), int(splits), _p(part), slopes, sinks, gt, _p(out),
-                                               _stream()))
+                                               terms.chunk, ctypes.c_float(terms.scale), int(splits), _p(part), slopes, sinks,
+                                               gt, int(terms.logistic), _p(terms.score_bias), _p(out), _stream()))
     elif fast and k_new is not None and vt_new is not None:
         B = n_cached.shape[0]
         n_tiles = int(sum(-(-int(x) // PREFILL_BLOCK) for x in ctx.host["n_new"]))
@@ -501,8 +603,9 @@ def attention_scored(q, k_new, v_new, pages, nkv: int, dv: int, table, ring_page
         _check(lib().tl_attn_prefill_terms_bf16(_p(q), _p(k_new), _p(vt_new), vt_new.shape[2], _p(ctx.tile_off), _p(pages),
                                                 _p(table), table.shape[1], ring_pages, _p(ctx.row_pos),
                                                 _p(ctx.cu_seqlens), _p(n_cached), B, n_tiles, nq, nkv, dk,
-                                                int(terms.window or 0), int(terms.keep_first or 0),
-                                                ctypes.c_float(terms.scale), slopes, sinks, gt, _p(out), _stream()))
+                                                int(terms.window or 0), int(terms.keep_first or 0), terms.chunk,
+                                                ctypes.c_float(terms.scale), slopes, sinks, gt, int(terms.logistic),
+                                                _p(terms.score_bias), _p(out), _stream()))
     else:
         attn_scored_plain(q, k_new, v_new, pages, nkv, dv, table, ring_pages, ctx.row_seq, ctx.row_pos,
                           ctx.cu_seqlens, n_cached, terms, gate, out)
@@ -675,11 +778,15 @@ class HeadTerms:
     attention itself, head by head (`head_prepare`): `bias` (float32 over the whole row, or None);
     `q_norm`, `k_norm` (float32 [dk] each, or None): every head divided by its own root mean
     square (eps inside the root) times a weight that all heads share; `mix`: 0, or 1 (the values
-    are left, unrounded, for later layers) or 2 (v <- (1 - lam) v + lam * the values that were left)."""
+    are left, unrounded, for later layers) or 2 (v <- (1 - lam) v + lam * the values that were left);
+    `unit_norm`: instead of the weighted norm, every head of q and of k is divided by its root mean
+    square (the same eps) AFTER the rotation, with no weight."""
 
-    def __init__(self, bias=None, q_norm=None, k_norm=None, eps: float = 0.0, mix: int = 0, lam: float = 0.0):
+    def __init__(self, bias=None, q_norm=None, k_norm=None, eps: float = 0.0, mix: int = 0, lam: float = 0.0,
+                 unit_norm: bool = False):
         self.bias, self.q_norm, self.k_norm, self.eps = bias, q_norm, k_norm, float(eps)
         self.mix, self.lam = int(mix), float(lam)
+        self.unit_norm = bool(unit_norm)
 
 
 def head_prepare(proj: torch.Tensor, row_pos, rotation, terms: HeadTerms, nq: int, nkv: int, dk: int, dv: int, ng: int,
@@ -688,7 +795,8 @@ def head_prepare(proj: torch.Tensor, row_pos, rotation, terms: HeadTerms, nq: in
     `gate` float32 [n, ng] (after the logistic function) and k [n, nkv, dk] and v [n, nkv, dv], or,
     with `pages` (one token a sequence, row n belongs to sequence n), k and v straight into the
     page of the row's position.  `v_first` (float32 [n, nkv*dv]): where a layer that mixes values
-    leaves or finds the first such layer's."""
+    leaves or finds the first such layer's.  nkv 0: the row holds [q | g] alone (a mixer that reads
+    another's keys and values)."""
     n = proj.shape[0]
     width = nq * dk + nkv * (dk + dv) + ng
     rot = _rotation(rotation, dk, "head_prepare")
@@ -707,7 +815,9 @@ def head_prepare(proj: torch.Tensor, row_pos, rotation, terms: HeadTerms, nq: in
             raise KernelError("head_prepare: mixing values needs the buffer they are left in")
         _req(v_first, "head_prepare.v_first", torch.float32, (n, nkv * dv))
     stride = 0
-    if pages is None:
+    if nkv == 0:
+        pages = k = v = None
+    elif pages is None:
         _req(k, "head_prepare.k", q.dtype, (n, nkv, dk))
         _req(v, "head_prepare.v", q.dtype, (n, nkv, dv))
     else:
@@ -717,8 +827,8 @@ def head_prepare(proj: torch.Tensor, row_pos, rotation, terms: HeadTerms, nq: in
             raise KernelError("head_prepare: pages of q's dtype and a page table with one row per row")
         stride = table.shape[1]
     _check(lib().tl_head_prepare(_p(proj), _p(row_pos), _p(rot.inv_freq), rot.rotary_dim, _p(terms.bias), _p(terms.q_norm),
-                                 _p(terms.k_norm), ctypes.c_float(terms.eps), terms.mix, ctypes.c_float(terms.lam),
-                                 _p(v_first) if terms.mix else None, n, nq, nkv, dk, dv, ng, _p(q),
+                                 _p(terms.k_norm), ctypes.c_float(terms.eps), int(terms.unit_norm), terms.mix,
+                                 ctypes.c_float(terms.lam), _p(v_first) if terms.mix else None, n, nq, nkv, dk, dv, ng, _p(q),
                                  _p(k) if pages is None else None, _p(v) if pages is None else None, _p(gate),
                                  _code(q.dtype), _p(table), stride, int(ring_pages), _p(pages), _stream()))
 
@@ -794,8 +904,9 @@ EXPERT_ACTIVATIONS = {"relu2": 0, "relu": 1}
 
 
 def route(h: torch.Tensor, router: torch.Tensor, groups: int, keep: int, top: int, weights: torch.Tensor,
-          chosen: Optional[torch.Tensor] = None) -> None:
-    """The router of a mixture of experts, in float32: s = softmax(router h) over the E experts; of the `keep`
+          chosen: Optional[torch.Tensor] = None, logistic: bool = False) -> None:
+    """The router of a mixture of experts, in float32: s = softmax(router h) over the E experts (`logistic`:
+    every expert's own 1 / (1 + exp(-router h)) instead); of the `keep`
     groups (of `groups` equal groups of neighbours; 0: no groups) whose best s is largest, the `top` experts
     with the largest s; `weights` float32 [n, E] receives s for those and 0 for the others, `chosen` (int32
     [n, top], or None) their indices, the best first."""
@@ -806,8 +917,54 @@ def route(h: torch.Tensor, router: torch.Tensor, groups: int, keep: int, top: in
     _req(weights, "route.weights", torch.float32, (n, E))
     if chosen is not None:
         _req(chosen, "route.chosen", torch.int32, (n, top))
-    _check(lib().tl_route(_p(h), _code(h.dtype), n, W, _p(router), E, int(groups), int(keep), int(top), _p(weights),
-                          _p(chosen), _stream()))
+    _check(lib().tl_route(_p(h), _code(h.dtype), n, W, _p(router), E, int(groups), int(keep), int(top), int(bool(logistic)),
+                          _p(weights), _p(chosen), _stream()))
+
+
+class GateTerms:
+    """The constants of a gated expert, act(g, u) = g' logistic(alpha g') (u' + shift) with g' = min(g, limit) and
+    u' = clamp(u, -limit, limit); the shared expert has a limit of its own (`limit_shared`; None: the same).
+    `on_input`: the router's weight multiplies the expert's input (g and u before the clamps) instead of its output."""
+
+    def __init__(self, limit: float, alpha: float, shift: float, limit_shared: Optional[float] = None, on_input: bool = False):
+        self.limit, self.alpha, self.shift = float(limit), float(alpha), float(shift)
+        self.limit_shared = self.limit if limit_shared is None else float(limit_shared)
+        self.on_input = bool(on_input)
+
+    def args(self):
+        return (ctypes.c_float(self.limit), ctypes.c_float(self.limit_shared), ctypes.c_float(self.alpha),
+                ctypes.c_float(self.shift), int(self.on_input))
+
+
+def expert_gated_act(gu: torch.Tensor, weights: Optional[torch.Tensor], E: int, ff: int, shared: int, terms: GateTerms,
+                     out: torch.Tensor) -> None:
+    """The activations of gated experts laid side by side: gu float32 [n, 2 (E ff + shared)] holds, expert after
+    expert, [gate (ff) | up (ff)] and behind them the shared expert's [gate (shared) | up (shared)]; out
+    [n, E ff + shared] = act(g, u) with the row's weight of the column's expert (`weights` float32 [n, E]; the
+    shared part has weight 1; E 0: no weights)."""
+    n = gu.shape[0]
+    total = E * ff + shared
+    _req(gu, "expert_gated_act.gu", torch.float32, (n, 2 * total))
+    if E:
+        _req(weights, "expert_gated_act.weights", torch.float32, (n, E))
+    _req(out, "expert_gated_act.out", None, (n, total))
+    _check(lib().tl_expert_gated_act(_p(gu), _p(weights) if E else None, n, int(E), int(ff), int(shared), *terms.args(),
+                                     _p(out), _code(out.dtype), _stream()))
+
+
+def expert_rows_gated_up(y: torch.Tensor, up: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor, ff: int, shared: int,
+                         terms: GateTerms, hs: torch.Tensor) -> None:
+    """The chosen gated experts' first halves, row by row (see `expert_rows_up`): up [2 (E ff + shared), H] is the
+    stacked matrix of `expert_gated_act`'s layout."""
+    n, H = y.shape
+    top, E = chosen.shape[1], weights.shape[1]
+    _req(y, "expert_rows_gated_up.y")
+    _req(up, "expert_rows_gated_up.up", y.dtype, (2 * (E * ff + shared), H))
+    _req(chosen, "expert_rows_gated_up.chosen", torch.int32, (n, top))
+    _req(weights, "expert_rows_gated_up.weights", torch.float32, (n, E))
+    _req(hs, "expert_rows_gated_up.hs", y.dtype, (n, top * ff + shared))
+    _check(lib().tl_expert_rows_gated_up(_p(y), H, _p(up), _p(chosen), _p(weights), n, E, top, int(ff), int(shared),
+                                         *terms.args(), _p(hs), _code(y.dtype), _stream()))
 
 
 def expert_act(u: torch.Tensor, weights: Optional[torch.Tensor], E: int, ff: int, activation: str, out: torch.Tensor) -> None:

@@ -7,6 +7,7 @@ from . import mistral as _mistral         # registers MistralForCausalLM
 from . import sozetar as _sozetar         # registers Sozetar
 from . import fanitar as _fanitar         # registers Fanitar
 from . import nepisun as _nepisun         # registers Nepisun
+from . import giforax as _giforax         # registers Giforax
 
 
 def model_spec_for(cfg: ModelConfig):

@@ -216,21 +216,31 @@ class ScoredAttentionMixer(Mixer):
 
 
 def attend_and_commit(ctx, run, q: torch.Tensor, k, v, nkv: int, dk: int, dv: int, terms, gate, att: torch.Tensor,
-                      tag: str = "") -> None:
-    """The attention of a step for a mixer that owns its keys and values and has made q [n, nq, dk]
-    and, unless every sequence brings one token (k and v are then None and lie in their pages
-    already), this step's k [n, nkv, dk] and v [n, nkv, dv]: the step's rows attend to the pages
-    for cached positions and to k and v for the new ones (values transposed by tiles where the
-    matrix cores run), and k and v are committed to the pages afterwards.  Scores with no term but the
-    scale and the window go through the kernels of the attention without terms where the matrix cores
-    take the shape (one product with the values instead of two, and the keys of few rows over a long
-    context cut into runs)."""
+                      tag: str = "", own: bool = True) -> None:
+    """The attention of a step for a mixer that has made q [n, nq, dk] and, unless every sequence
+    brings one token (k and v are then None and lie in their pages already), this step's
+    k [n, nkv, dk] and v [n, nkv, dv]: the step's rows attend to the pages for cached positions and
+    to k and v for the new ones (values transposed by tiles where the matrix cores run), and k and
+    v are committed to the pages afterwards.  Scores with no term but the scale and the window go
+    through the kernels of the attention without terms where the matrix cores take the shape (one
+    product with the values instead of two, and the keys of few rows over a long context cut into
+    runs).  A run whose keys a later run reads (`run.kv_read_later`) leaves its new rows in
+    `ctx.host["kv_new_<run>"]` and commits at the end of the step (the later run still reads the
+    ring's old rows); its k and v must then be buffers that no other run writes.  `own` False: the
+    run reads the keys and values of `run.kv_source` (k and v are ignored) and commits nothing."""
     group = run.kv_group
     pages = group.storage[run.kv_layer]
     table = ctx.tables[run.kv_group_index]
     cores = ops.scored_on_matrix_cores(ctx.dtype, dk, dv) and pages.dim() == 5
     bare = (cores and terms.slopes is None and terms.sinks is None and gate is None and not terms.keep_first
-            and att.dtype == ctx.dtype)
+            and not terms.chunk and not terms.logistic and att.dtype == ctx.dtype)
+    if not own and not ctx.all_single:
+        k, v, vt = ctx.host[f"kv_new_{run.kv_source}"]
+        if vt is None and cores:
+            raise RuntimeError("attention: the run that owns the keys left no transposed values")
+        ops.attention_scored(q, k, v, pages, nkv, dv, table, group.ring_pages, ctx, ctx.len_before, terms, gate, att,
+                             vt_new=vt)
+        return
     if ctx.all_single:
         if bare:
             ops.attention(q, None, None, pages, table, group.ring_pages, ctx, ctx.len_after, terms.window, terms.scale, att)
@@ -248,11 +258,19 @@ def attend_and_commit(ctx, run, q: torch.Tensor, k, v, nkv: int, dk: int, dv: in
     else:
         ops.attention_scored(q, k, v, pages, nkv, dv, table, group.ring_pages, ctx, ctx.len_before, terms, gate, att,
                              vt_new=vt)
-    if vt is not None and pages.dim() == 5:       # values a tile at a time, in whole lines
-        ops.kv_commit_tiles(k, vt, ctx.row_seq, ctx.row_pos, ctx.tile_off, ctx.len_before, ctx.len_after, table,
-                            group.ring_pages, pages)
+
+    def commit():
+        if vt is not None and pages.dim() == 5:       # values a tile at a time, in whole lines
+            ops.kv_commit_tiles(k, vt, ctx.row_seq, ctx.row_pos, ctx.tile_off, ctx.len_before, ctx.len_after, table,
+                                group.ring_pages, pages)
+        else:
+            ops.kv_commit_wide(k, v, ctx.row_seq, ctx.row_pos, ctx.len_after, table, group.ring_pages, pages)
+
+    if run.kv_read_later:
+        ctx.host[f"kv_new_{run.index}"] = (k, v, vt)
+        ctx.host.setdefault("deferred", []).append(commit)
     else:
-        ops.kv_commit_wide(k, v, ctx.row_seq, ctx.row_pos, ctx.len_after, table, group.ring_pages, pages)
+        commit()
 
 
 register_part("mixer", "scored_attention", ScoredAttentionMixer)

@@ -95,6 +95,9 @@ class ModelSpec:
     ignore_tensors: Tuple[str, ...] = ()
     # parts of category "stream" that change the stream between runs (`Run.entry`): (name prefix, spec)
     stream_parts: List[Tuple[str, PartSpec]] = field(default_factory=list)
+    # (index into `stream_parts`, t): that part changes the stream once more after the last run, before the
+    # final norm
+    exit: Optional[Tuple[int, int]] = None
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
         """Every tensor name the model binds, in a fixed order."""

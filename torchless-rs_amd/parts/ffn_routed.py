@@ -9,6 +9,11 @@ more product, in float32: s = softmax(W_r y) over all experts.  The experts form
 the `group_keep` best groups can be chosen (no groups: any expert).  The `top` experts with the
 largest s are chosen; the result is the sum of their outputs weighted by their s, not
 renormalised, plus a shared expert's (`shared_size`; None: none) that runs for every token.
+`score` "sigmoid" makes every expert's score its own logistic function of the router's product
+instead of a softmax over the experts.  `gated` experts have a gate beside the up projection,
+down(act(gate t, up t)) with the clamped activation of `ops.GateTerms` (`activation_constants`:
+limit, alpha, shift; the shared expert's limit may differ, `shared_limit`), and `weight_on`
+"input" multiplies an expert's INPUT t = s y by the router's weight instead of its output.
 
 All experts run as ONE wide feed-forward: their up projections stacked by rows (the shared
 expert's behind them), the activation times the row's weight of the column's expert, which is
@@ -91,13 +96,32 @@ class RoutedExperts(FeedForward):
 
     # leaf names under `prefix`; "{e}" is the expert's number
     NAMES = {"router": "router", "up": "e{e}.up", "down": "e{e}.down", "shared_up": "shared.up",
-             "shared_down": "shared.down"}
+             "shared_down": "shared.down", "gate": "e{e}.gate", "shared_gate": "shared.gate"}
+    SCORES = ("softmax", "sigmoid")
+    GATED_ACTIVATION = "swish_clamped"
 
     def __init__(self, hidden_size: int, n_experts: int, top: int, expert_size: int, group_count: Optional[int] = None,
                  group_keep: Optional[int] = None, shared_size: Optional[int] = None, activation: str = "relu2",
-                 prefix: str = "mlp.", names: Optional[Dict[str, str]] = None):
-        if activation not in ops.EXPERT_ACTIVATIONS:
+                 prefix: str = "mlp.", names: Optional[Dict[str, str]] = None, score: str = "softmax",
+                 gated: bool = False, activation_constants: Optional[Dict[str, float]] = None,
+                 shared_limit: Optional[float] = None, weight_on: str = "output"):
+        self.gated = bool(gated)
+        if score not in self.SCORES:
+            raise ValueError(f"experts: scores are one of {self.SCORES}, got {score!r}")
+        if weight_on not in ("output", "input"):
+            raise ValueError(f"experts: the router's weight is on an expert's 'output' or 'input', got {weight_on!r}")
+        if self.gated:
+            need = {"limit", "alpha", "shift"}
+            if activation != self.GATED_ACTIVATION or set(activation_constants or {}) != need:
+                raise ValueError(f"experts: gated experts have the activation {self.GATED_ACTIVATION!r} with the "
+                                 f"constants {sorted(need)}, got {activation!r} with {sorted(activation_constants or {})}")
+            c = activation_constants
+            self.gate_terms = ops.GateTerms(c["limit"], c["alpha"], c["shift"], shared_limit, weight_on == "input")
+        elif activation not in ops.EXPERT_ACTIVATIONS:
             raise ValueError(f"experts: no activation {activation!r}; there are {sorted(ops.EXPERT_ACTIVATIONS)}")
+        elif weight_on != "output" or activation_constants or shared_limit is not None:
+            raise ValueError("experts: the weight on the input, constants and a shared limit go with gated experts")
+        self.logistic = score == "sigmoid"
         if not (1 <= top <= n_experts):
             raise ValueError(f"experts: {top} of {n_experts}")
         if group_count:
@@ -118,24 +142,30 @@ class RoutedExperts(FeedForward):
         p, nm = self.prefix, self.names
         out: Dict[str, WeightSpec] = {}
         for e in range(self.E):
+            if self.gated:
+                out[p + nm["gate"].format(e=e)] = WeightSpec((self.ff, self.H))
             out[p + nm["up"].format(e=e)] = WeightSpec((self.ff, self.H))
             out[p + nm["down"].format(e=e)] = WeightSpec((self.H, self.ff))
         out[p + nm["router"]] = WeightSpec((self.E, self.H))
         if self.shared:
+            if self.gated:
+                out[p + nm["shared_gate"]] = WeightSpec((self.shared, self.H))
             out[p + nm["shared_up"]] = WeightSpec((self.shared, self.H))
             out[p + nm["shared_down"]] = WeightSpec((self.H, self.shared))
         return out
 
     def load(self, tensors, compute_dtype) -> None:
         p, nm = self.prefix, self.names
-        ups = [tensors[p + nm["up"].format(e=e)] for e in range(self.E)]
+        ups = []
+        for e in range(self.E):          # a gated expert's rows: [gate | up]
+            ups += ([tensors[p + nm["gate"].format(e=e)]] if self.gated else []) + [tensors[p + nm["up"].format(e=e)]]
         downs = [tensors[p + nm["down"].format(e=e)] for e in range(self.E)]
         if self.shared:
-            ups.append(tensors[p + nm["shared_up"]])
+            ups += ([tensors[p + nm["shared_gate"]]] if self.gated else []) + [tensors[p + nm["shared_up"]]]
             downs.append(tensors[p + nm["shared_down"]])
         if len({w.dtype for w in ups + downs}) > 1:
             ups, downs = [w.to(torch.float32) for w in ups], [w.to(torch.float32) for w in downs]
-        self.up = Linear(torch.cat(ups, dim=0), tiled=True)          # [E * ff + shared, H]
+        self.up = Linear(torch.cat(ups, dim=0), tiled=True)          # [E * ff + shared, H]; gated: twice the rows
         self.down = Linear(torch.cat(downs, dim=1), tiled=True)      # [H, E * ff + shared]
         self.router = tensors[p + nm["router"]].to(torch.float32).contiguous()
 
@@ -148,9 +178,12 @@ class RoutedExperts(FeedForward):
         ws = ctx.workspace
         weights = ws.get("experts_w", (n, self.E), torch.float32)
         chosen = ws.get("experts_chosen", (n, self.top), torch.int32)
-        ops.route(y, self.router, self.groups, self.keep, self.top, weights, chosen)
+        ops.route(y, self.router, self.groups, self.keep, self.top, weights, chosen, logistic=self.logistic)
         hs = ws.get("experts_hs", (n, self.top * self.ff + self.shared), y.dtype)
-        ops.expert_rows_up(y, self.up.weight, chosen, weights, self.ff, self.shared, self.activation, hs)
+        if self.gated:
+            ops.expert_rows_gated_up(y, self.up.weight, chosen, weights, self.ff, self.shared, self.gate_terms, hs)
+        else:
+            ops.expert_rows_up(y, self.up.weight, chosen, weights, self.ff, self.shared, self.activation, hs)
         ops.expert_rows_down(hs, self.down.weight, chosen, self.E, self.ff, self.shared, out, accumulate)
 
     def many_rows(self, ctx, y: torch.Tensor) -> bool:
@@ -165,7 +198,7 @@ class RoutedExperts(FeedForward):
         ws = ctx.workspace
         weights = ws.get("experts_w", (n, E), torch.float32)
         chosen = ws.get("experts_chosen", (n, top), torch.int32)
-        ops.route(y, self.router, self.groups, self.keep, self.top, weights, chosen)
+        ops.route(y, self.router, self.groups, self.keep, self.top, weights, chosen, logistic=self.logistic)
         flat = chosen.view(-1).long()
         order = torch.argsort(flat, stable=True)                       # pairs by expert, a row's place kept within one
         counts = torch.bincount(flat, minlength=E).tolist()            # (the host waits for the router here)
@@ -173,14 +206,18 @@ class RoutedExperts(FeedForward):
         ys = y.index_select(0, rows)                                   # [n * top, H]
         scale = weights.gather(1, chosen.long()).view(-1).index_select(0, order).view(-1, 1).contiguous()
         up_w, down_w = self.up.weight, self.down.weight
-        u = ws.get("experts_gu", (n * top, ff), torch.float32)
+        wide = 2 if self.gated else 1               # a gated expert's rows are [gate | up]
+        u = ws.get("experts_gu", (n * top, wide * ff), torch.float32)
         at = 0
         for e, c in enumerate(counts):
             if c:
-                ops.gemm(ys[at:at + c], up_w[e * ff:(e + 1) * ff], u[at:at + c])
+                ops.gemm(ys[at:at + c], up_w[wide * e * ff:wide * (e + 1) * ff], u[at:at + c])
                 at += c
         h = ws.get("experts_gh", (n * top, ff), y.dtype)
-        ops.expert_act(u, scale, 1, ff, self.activation, h)
+        if self.gated:
+            ops.expert_gated_act(u, scale, 1, ff, 0, self.gate_terms, h)
+        else:
+            ops.expert_act(u, scale, 1, ff, self.activation, h)
         z = ws.get("experts_gz", (n * top, H), torch.float32)
         at = 0
         for e, c in enumerate(counts):
@@ -191,10 +228,13 @@ class RoutedExperts(FeedForward):
         back[order] = torch.arange(n * top, device=order.device)
         total = z.index_select(0, back).view(n, top, H).sum(dim=1)     # a row's experts in the order it chose them
         if self.shared:
-            us = ws.get("experts_su", (n, self.shared), torch.float32)
-            ops.gemm(y, up_w[E * ff:], us)
+            us = ws.get("experts_su", (n, wide * self.shared), torch.float32)
+            ops.gemm(y, up_w[wide * E * ff:], us)
             hs = ws.get("experts_sh", (n, self.shared), y.dtype)
-            ops.expert_act(us, None, 0, self.shared, self.activation, hs)
+            if self.gated:
+                ops.expert_gated_act(us, None, 0, 0, self.shared, self.gate_terms, hs)
+            else:
+                ops.expert_act(us, None, 0, self.shared, self.activation, hs)
             total.add_(torch.mm(hs, down_w[:, E * ff:].t(), out_dtype=torch.float32))
         if accumulate:
             out.add_(total)
@@ -205,11 +245,14 @@ class RoutedExperts(FeedForward):
         n = y.shape[0]
         ws = ctx.workspace
         weights = ws.get("experts_w", (n, self.E), torch.float32)
-        ops.route(y, self.router, self.groups, self.keep, self.top, weights)
-        u = ws.get("experts_u", (n, self.total), torch.float32)
+        ops.route(y, self.router, self.groups, self.keep, self.top, weights, logistic=self.logistic)
+        u = ws.get("experts_u", (n, (2 if self.gated else 1) * self.total), torch.float32)
         self.up(y, u)
         h = ws.get("experts_h", (n, self.total), ctx.dtype)
-        ops.expert_act(u, weights, self.E, self.ff, self.activation, h)
+        if self.gated:
+            ops.expert_gated_act(u, weights, self.E, self.ff, self.shared, self.gate_terms, h)
+        else:
+            ops.expert_act(u, weights, self.E, self.ff, self.activation, h)
         return h
 
     def forward(self, ctx, y: torch.Tensor, x: torch.Tensor) -> None:

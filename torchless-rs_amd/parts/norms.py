@@ -1,8 +1,8 @@
 """Norms over a row of the stream, in float32.
 
 RMSNorm: y = x / sqrt(mean(x^2) + eps) * w (src/kernels/mod.rs:558-568 of the
-reference; weight used as it is).  LayerNorm: y = (x - mean) / sqrt(var + eps) * w
-with var the mean of the squared deviations, a weight and no bias."""
+reference; weight used as it is).  LayerNorm: y = (x - mean) / sqrt(var + eps) * w + b
+with var the mean of the squared deviations, a weight and an optional bias."""
 from __future__ import annotations
 
 from typing import Dict
@@ -66,33 +66,50 @@ class RMSNorm(Norm):
 
 
 class LayerNorm(Norm):
-    """Mean and variance over the row; a weight, no bias.  Besides the plain `forward` it can
-    be the norm of a sublayer's OUTPUT (`add_to`): x += norm(z), in one kernel that also
-    leaves the new stream in the compute dtype for the product that reads it next."""
+    """Mean and variance over the row; a weight and, with `bias_name`, a bias of the norm's own.
+    Besides the plain `forward` it can be the norm of a sublayer's OUTPUT (`add_to`): x += norm(z),
+    in one kernel that also leaves the new stream in the compute dtype for the product that reads
+    it next, or (`then`) runs the layer norm that reads the stream next on the new row."""
     graph_safe = True
 
-    def __init__(self, size: int, eps: float, name: str = "weight"):
-        """`name`: the weight's leaf name behind the norm's prefix ("" where the prefix is the tensor)."""
+    def __init__(self, size: int, eps: float, name: str = "weight", bias_name: str = None):
+        """`name`: the weight's leaf name behind the norm's prefix ("" where the prefix is the tensor);
+        `bias_name`: the bias's (None: the norm has none)."""
         self.size = int(size)
         self.eps = float(eps)
         self.name = name
-        self.weight = None
+        self.bias_name = bias_name
+        self.weight = self.beta = None
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
-        return {self.name: WeightSpec((self.size,), init="ones")}
+        out = {self.name: WeightSpec((self.size,), init="ones")}
+        if self.bias_name is not None:
+            out[self.bias_name] = WeightSpec((self.size,))
+        return out
 
     def load(self, tensors, compute_dtype) -> None:
         self.weight = tensors[self.name].to(torch.float32).contiguous()
+        if self.bias_name is not None:
+            self.beta = tensors[self.bias_name].to(torch.float32).contiguous()
 
     def forward(self, ctx, x: torch.Tensor, out: torch.Tensor) -> None:
         flush = getattr(ctx, "pending", None)
         if flush is not None:
             ops.add_partials(x, flush)
             ctx.pending = None
-        ops.layernorm(x, self.weight, self.eps, out)
+        ops.layernorm(x, self.weight, self.eps, out, beta=self.beta)
 
     def add_to(self, ctx, z: torch.Tensor, x: torch.Tensor, out=None, bias=None, then=None) -> None:
-        ops.layernorm(z, self.weight, self.eps, out, add_to=x, bias=bias)
+        nxt = then[0] if then is not None and isinstance(then[0], LayerNorm) and then[0].size == self.size else None
+        if out is None and ops.layernorm_rows_in_registers(self.size):
+            if nxt is not None:
+                ops.layernorm_add_norm(z, self.weight, self.beta, self.eps, x, bias=bias, w_next=nxt.weight,
+                                       beta_next=nxt.beta, eps_next=nxt.eps, out=then[1])
+                ctx.prenormed = (nxt, then[1], None)
+            else:
+                ops.layernorm_add_norm(z, self.weight, self.beta, self.eps, x, bias=bias)
+            return
+        ops.layernorm(z, self.weight, self.eps, out, add_to=x, bias=bias, beta=self.beta)
 
 
 register_part("norm", "rmsnorm", RMSNorm)

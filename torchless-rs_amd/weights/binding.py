@@ -26,7 +26,7 @@ class WeightSpec:
     """What a part expects under one name."""
     shape: Tuple[int, ...]
     integer: bool = False
-    init: str = "normal"      # how random weights fill it: "normal" or "ones" (norm weights)
+    init: str = "normal"      # how random weights fill it: "normal", "ones" (norm weights) or "mean" (weights of an average)
 
 
 class WeightBindingError(ValueError):

@@ -34,6 +34,11 @@ def random_tensors(expected: Dict[str, WeightSpec], seed: int, std: float = 0.02
                 t += norm_std * torch.randn(spec.shape, generator=gen, dtype=torch.float32,
                                             device=device)
             out[name] = t.to(dtype)
+        elif spec.init == "mean":       # weights of an average: 1 / their number each, so that a random model's stream keeps its size
+            t = torch.full(spec.shape, 1.0 / max(1, spec.shape[-1] if spec.shape else 1), dtype=torch.float32, device=device)
+            if norm_std:
+                t += norm_std * torch.randn(spec.shape, generator=gen, dtype=torch.float32, device=device) / max(1, t.numel())
+            out[name] = t.to(dtype)
         else:
             t = torch.randn(spec.shape, generator=gen, dtype=torch.float32, device=device)
             out[name] = t.mul_(std).to(dtype)
