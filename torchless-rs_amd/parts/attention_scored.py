@@ -266,7 +266,7 @@ def attend_and_commit(ctx, run, q: torch.Tensor, k, v, nkv: int, dk: int, dv: in
         else:
             ops.kv_commit_wide(k, v, ctx.row_seq, ctx.row_pos, ctx.len_after, table, group.ring_pages, pages)
 
-    if run.kv_read_later:
+    if getattr(run, "kv_read_later", False):
         ctx.host[f"kv_new_{run.index}"] = (k, v, vt)
         ctx.host.setdefault("deferred", []).append(commit)
     else:
