@@ -176,6 +176,66 @@ def nepisun_counts(z: dict, layers: int, B: int, C: int, T: int):
     return w, kv, att, w_read
 
 
+def giforax_layers(layers: int):
+    """The mixers of `giforax_config(z, layers)`: attention with keys of its own, attention that reads the first
+    layer's keys, a gated recurrence, attention, and so on; every layer has a routed feed-forward."""
+    kinds = ["attention", "reader", "mingru", "attention"]
+    return [kinds[i % 4] if i else "attention" for i in range(layers)]
+
+
+def giforax_sizes(z: dict):
+    """Sizes of the Giforax layers at the layer sizes `z`: a recurrence as wide as the model; 16 gated experts of an
+    eighth of the dense feed-forward's hidden size of which a token uses 4, beside a shared one of half of it: a
+    token multiplies as much as in the dense gated feed-forward.  Chunks as long as the other designs' window."""
+    return dict(gru=z["width"], experts=16, top=4, expert_ff=z["ff"] // 8, shared_ff=z["ff"] // 2, chunk=z["window"])
+
+
+def giforax_config(z: dict, layers: int):
+    """config.json of a Giforax model with the layer sizes `z` (see `giforax_layers`, `giforax_sizes`)."""
+    n = giforax_sizes(z)
+    out = []
+    for mix in giforax_layers(layers):
+        if mix == "mingru":
+            kind, m = "mingru", {"width": n["gru"]}
+        else:
+            kind = "attention"
+            m = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"], "scale": z["dim"] ** -0.5,
+                 "rot": {"base": 10000.0, "dims": z["dim"] // 2}}
+            if n["chunk"]:
+                m["mask"] = {"size": n["chunk"]}
+            if mix == "reader":
+                m["kv_from"] = 0
+        mlp = {"kind": "moe", "router": {"experts": n["experts"], "top": n["top"]},
+               "expert": {"ff": n["expert_ff"], "limit": 7.0}, "shared": {"ff": n["shared_ff"], "limit": 7.0}}
+        out.append({"type": kind, "mixer": m, "mlp": mlp})
+    return {"architecture": "Giforax", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6},
+            "embedding": {"scale": 1.0}, "layers": out}
+
+
+def giforax_counts(z: dict, layers: int, B: int, C: int, T: int):
+    """(weight elements that a prompt's products multiply a row by, bytes of keys, values and recurrent state that a
+    decode step reads and writes, multiply-adds times two of a prompt's attention, weight elements that a decode step
+    of B rows must read) of `giforax_config(z, layers)`.  A position sees the keys of its own chunk alone; a routed
+    feed-forward multiplies a row by its `top` experts and the shared one, and a decode step reads the experts that B
+    rows can choose at most."""
+    H, nq, nkv, d = z["width"], z["heads"], z["kv_heads"], z["dim"]
+    n = giforax_sizes(z)
+    chunk = n["chunk"]
+    w = w_read = kv = att = 0
+    for mix in giforax_layers(layers):
+        if mix == "mingru":
+            m = 4 * n["gru"] * H
+            kv += B * n["gru"] * 4 * 2
+        else:
+            m = 2 * nq * d * H + nq * H + (2 * nkv * d * H if mix == "attention" else 0)
+            seen = ((C - 1) % chunk + 1) if chunk else C
+            kv += B * seen * nkv * 2 * d * 2
+            att += 4 * nq * d * sum((p % chunk if chunk else p) + 1 for p in range(T))
+        w += m + 3 * H * (n["top"] * n["expert_ff"] + n["shared_ff"]) + n["experts"] * H
+        w_read += m + 3 * H * (min(n["experts"], B * n["top"]) * n["expert_ff"] + n["shared_ff"]) + n["experts"] * H
+    return w, kv, att, w_read
+
+
 def bench_designs(args) -> int:
     """Prefill (one prompt of --prefill-tokens in one step) and decode (--batch sequences at --context
     positions, one token a step through captured graphs) of the three designs at equal layer sizes,
@@ -259,6 +319,8 @@ def bench_designs(args) -> int:
             row["fanitar"] = measure(fanitar_config(z, L), z, counts=fanitar_counts(z, L, B, C, T))
         if "nepisun" in which:
             row["nepisun"] = measure(nepisun_config(z, L), z, counts=nepisun_counts(z, L, B, C, T))
+        if "giforax" in which:
+            row["giforax"] = measure(giforax_config(z, L), z, counts=giforax_counts(z, L, B, C, T))
         if "sozetar" in which:
             row["sozetar"] = measure(soz, z)
         if "mistral" in which:
@@ -293,10 +355,10 @@ def main() -> int:
     ap.add_argument("--only", choices=["prefill", "decode", "pipes", "designs"], default=None,
                     help="measure one phase only and print its line to stderr (for profiling); pipes: whether a "
                          "SIMD's matrix and vector pipes overlap (ops.measure_pipes); designs: prefill and decode of "
-                         "the Fanitar, Sozetar and Nepisun designs beside the Mistral design at equal layer sizes (--design-sizes, "
+                         "the Fanitar, Sozetar, Nepisun and Giforax designs beside the Mistral design at equal layer sizes (--design-sizes, "
                          "--layers, --batch, --context, --prefill-tokens apply)")
     ap.add_argument("--design-names", default="fanitar,sozetar,mistral",
-                    help="with --only designs: which designs to run (of fanitar, sozetar, nepisun, mistral)")
+                    help="with --only designs: which designs to run (of fanitar, sozetar, nepisun, giforax, mistral)")
     ap.add_argument("--design-sizes", default="2b,7b,12b",
                     help="with --only designs: which layer sizes to run (of %s)" % ",".join(sorted(DESIGN_SIZES)))
     args = ap.parse_args()

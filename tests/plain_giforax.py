@@ -102,14 +102,20 @@ def gated_expert(h, w, p, limit):
 def route(h, w, p, r, margins=None):
     """Scores s = logistic(W_r h); the `top` largest are chosen (of equal ones the smaller index).
     Returns [T, E] weights: s where chosen, 0 elsewhere.  `margins`: a list that receives, per row,
-    the gap between the last chosen and the first not chosen score."""
-    s = torch.sigmoid(h @ w[p + "router"].T)
+    the gap between the last chosen and the first not chosen expert's product W_r h, as a share of
+    the root mean square of the row's products (infinite where every expert is chosen)."""
+    z = h @ w[p + "router"].T
+    s = torch.sigmoid(z)
     order = torch.sort(s, dim=-1, descending=True, stable=True)
     top = r["top"]
     out = torch.zeros_like(s)
     out.scatter_(1, order.indices[:, :top], order.values[:, :top])
     if margins is not None:
-        gap = (order.values[:, top - 1] - order.values[:, top]) if top < s.shape[1] else torch.full((s.shape[0],), math.inf, dtype=s.dtype)
+        if top < s.shape[1]:
+            zs = torch.gather(z, 1, order.indices)
+            gap = (zs[:, top - 1] - zs[:, top]) / torch.sqrt((z * z).mean(dim=-1) + 1e-30)
+        else:
+            gap = torch.full((s.shape[0],), math.inf, dtype=s.dtype)
         margins.append(gap)
     return out
 
