@@ -132,6 +132,39 @@ def test_the_weighted_sum_of_the_streams_versions():
             assert rel_err(x, want) < 1e-6, (n, H, t)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H", [30, 64, 2052])
+def test_the_weighted_sum_on_the_way_from_one_norm_to_the_next(dtype, H):
+    """x += norm(z); the new x is kept as version t and replaced by the weighted sum of the versions; the next norm
+    reads the sum: in one kernel where the row fits it, step by step where not, with the same results."""
+    from torchless_rs_amd.parts.norms import LayerNorm
+    g = torch.Generator().manual_seed(H + 1)
+    n, T = 6, 3
+    norms = []
+    for i in range(2):
+        ln = LayerNorm(H, 1e-5, name="", bias_name=".b")
+        ln.load({"": dev(1 + 0.3 * torch.randn(H, generator=g)), ".b": dev(torch.randn(H, generator=g))}, TORCH[dtype])
+        norms.append(ln)
+    a, b = norms
+    versions = torch.randn(T + 1, n, H, generator=g)
+    coef = torch.randn(T + 1, generator=g)
+    z, x = torch.randn(n, H, generator=g) * 2, torch.randn(n, H, generator=g)
+    new = x.double() + plain.layer_norm(z.double(), a.eps, a.weight.double().cpu(), a.beta.double().cpu())
+    want_x = coef[T].double() * new + sum(coef[j].double() * versions[j].double() for j in range(T))
+    want_y = plain.layer_norm(want_x, b.eps, b.weight.double().cpu(), b.beta.double().cpu())
+    for then in (None, "next"):
+        kept = dev(versions.clone())
+        kept[T] = float("nan")
+        xs, out = dev(x.clone()), torch.empty(n, H, dtype=TORCH[dtype], device="cuda")
+        ctx = step_ctx(dtype)
+        a.add_to(ctx, dev(z.clone()), xs, then=(b, out) if then else None, between=(kept, dev(coef), T))
+        assert rel_err(xs, want_x) < 1e-5 and rel_err(kept[T], new) < 1e-5
+        if then and H % 4 == 0:
+            assert ctx.prenormed[0] is b and rel_err(out, want_y) < (1e-5 if dtype == "float32" else 1e-2)
+        else:
+            assert ctx.prenormed is None
+
+
 # ---------------------------------------------------------------------------------------------
 # the gated recurrence
 # ---------------------------------------------------------------------------------------------
@@ -389,7 +422,7 @@ ATT_TOL = {"float32": 2e-5, "bfloat16": 1.2e-2}
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("chunk", [1, 2, 63, 64, 65, 100, 129, 200])
-@pytest.mark.parametrize("dk, dv", [(16, 8), (64, 64), (96, 96)])
+@pytest.mark.parametrize("dk, dv", [(16, 8), (48, 48), (64, 64), (96, 96)])
 def test_a_key_just_inside_and_just_outside_a_chunk(dtype, chunk, dk, dv):
     """Every key's own weight is a thousandth (a bias of -7) but for the keys at both sides of every chunk's edge, the
     last of a chunk and the first of the next, which every query scores at +9: a row's result is the values of those
@@ -424,7 +457,7 @@ def test_a_key_just_inside_and_just_outside_a_chunk(dtype, chunk, dk, dv):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("dk, dv", [(32, 16), (64, 64), (128, 128)])
+@pytest.mark.parametrize("dk, dv", [(32, 16), (64, 64), (80, 80), (128, 128), (256, 256)])
 def test_a_far_key_and_the_first_tokens(dtype, dk, dv):
     """No chunks (and one chunk of 1,000): position 3 is the one loud key among 700, seen from everywhere behind it, in a
     prompt, in portions and by single tokens."""
@@ -583,16 +616,18 @@ def test_the_stream_after_every_layer(zoo, name, dtype):
     model_ = load_model(z["dir"], dtype)
     eng = Engine(model_, max_tokens=256, use_graphs=False)
     seen = []
-    part = model_.stream_parts[0]
-    inner = part.forward
+    for blk in model_.blocks[1:]:            # what a layer reads is the stream as the layer before and the sum left it
+        inner = blk.forward
 
-    def spy(ctx, x, embedded, t):
-        inner(ctx, x, embedded, t)
-        if t > 0:
+        def spy(ctx, run, x, *a, _inner=inner, **kw):
             seen.append(x.clone())
-    part.forward = spy
+            _inner(ctx, run, x, *a, **kw)
+        blk.forward = spy
+    last = model_.final_norm.forward
+    model_.final_norm.forward = lambda ctx, xs, y: (seen.append(xs.clone()), last(ctx, xs, y))[1]
+    p = z["prompts"][2]
     s = eng.alloc()
-    eng.step([SeqInput(s, z["prompts"][2], [0])])
+    eng.step([SeqInput(s, p, list(range(len(p))))])
     eng.free(s)
     assert len(seen) == len(streams)
     for i, (got, want) in enumerate(zip(seen, streams)):
@@ -730,7 +765,7 @@ def test_a_long_prompt_goes_by_runs_and_many_rows_expert_by_expert(zoo, monkeypa
         got = eng.step([SeqInput(s, p, list(range(len(p))))]).clone()
         eng.free(s)
         assert calls and all(c == len(p) for c in calls), calls
-        assert runs and all(r == -(-len(p) // 64) for r in runs), runs
+        assert runs and all(r == -(-len(p) // ops.gated_recurrence_chunk()) for r in runs), runs
         close(got, z["want"][3], "bfloat16", (name, "expert by expert"), z["margin"][3])
         s = eng.alloc()                                                   # two unequal prompts in one step
         q = z["prompts"][2]

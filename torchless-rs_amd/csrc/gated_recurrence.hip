@@ -19,7 +19,7 @@
 
 namespace tl {
 
-constexpr int RC_CHUNK = 64;
+constexpr int RC_CHUNK = 32;
 
 __device__ __forceinline__ float logistic(float v) { return 1.0f / (1.0f + expf(-v)); }
 __device__ __forceinline__ float candidate(float u) { return u >= 0.f ? u + 0.5f : logistic(u); }
@@ -70,7 +70,7 @@ gru_chunks_kernel(const float* __restrict__ proj, const float* __restrict__ bz, 
   if (ch >= W || !run_of(blockIdx.y, cu_seqlens, B, b, first, r0, r1)) return;
   const float zb = bz ? bz[ch] : 0.f, xb = bx ? bx[ch] : 0.f;
   float p = 1.f, q = 0.f;
-#pragma unroll 4
+#pragma unroll 8
   for (int r = r0; r < r1; ++r) {
     const float* row = proj + (size_t)r * 3 * W;
     const float z = logistic(row[ch] + zb);
@@ -94,7 +94,7 @@ gru_apply_kernel(const float* __restrict__ proj, const float* __restrict__ bz, c
   float S = start[(size_t)b * W + ch];
   for (int i = first; i < (int)blockIdx.y; ++i) S = P[(size_t)i * W + ch] * S + Q[(size_t)i * W + ch];
   const float zb = bz ? bz[ch] : 0.f, xb = bx ? bx[ch] : 0.f;
-#pragma unroll 4
+#pragma unroll 8
   for (int r = r0; r < r1; ++r) {
     const float* row = proj + (size_t)r * 3 * W;
     const float z = logistic(row[ch] + zb);

@@ -10,7 +10,9 @@
 // stream, and the norm that reads the stream next runs on the new row in the same pass:
 //     x += LN(z + bias; w1, b1) ;  out = LN(x; w2, b2)        (the second part optional)
 // with LN(t; w, b) = (t - mean) / sqrt(mean((t - mean)^2) + eps) * w + b.  The row stays in
-// registers: one read of z and x, one write of x and out.
+// registers: one read of z and x, one write of x and out.  Between the two the weighted sum
+// above may take place on the row (`kept` given): the new x is kept as version t and replaced
+// by the sum, which the second norm then reads.
 #include "common.hpp"
 
 namespace tl {
@@ -47,7 +49,8 @@ template <typename TO, int IT>
 __global__ void __launch_bounds__(256)
 layernorm_add_norm_kernel(const float* __restrict__ z, const float* __restrict__ bias, const float* __restrict__ w1,
                           const float* __restrict__ b1, float eps1, float* __restrict__ x, const float* __restrict__ w2,
-                          const float* __restrict__ b2, float eps2, TO* __restrict__ out, int H) {
+                          const float* __restrict__ b2, float eps2, TO* __restrict__ out, int H, float* __restrict__ kept,
+                          const float* __restrict__ coef, int t, long long total) {
   __shared__ float sh[4];
   const int n = blockIdx.x;
   const int nv = H / 4;
@@ -98,6 +101,17 @@ layernorm_add_norm_kernel(const float* __restrict__ z, const float* __restrict__
       const float4 y = affine(v[i], sd1, w1, b1, c);
       float4 a = xr[c];
       a.x += y.x; a.y += y.y; a.z += y.z; a.w += y.w;
+      if (kept != nullptr) {                    // version t of the stream, and the weighted sum of versions 0 .. t
+        const long long at = (long long)n * H + 4 * c;
+        *reinterpret_cast<float4*>(kept + (long long)t * total + at) = a;
+        const float ct = coef[t];
+        a.x *= ct; a.y *= ct; a.z *= ct; a.w *= ct;
+        for (int j = t - 1; j >= 0; --j) {
+          const float4 k = *reinterpret_cast<const float4*>(kept + (long long)j * total + at);
+          const float cj = coef[j];
+          a.x = fmaf(cj, k.x, a.x); a.y = fmaf(cj, k.y, a.y); a.z = fmaf(cj, k.z, a.z); a.w = fmaf(cj, k.w, a.w);
+        }
+      }
       xr[c] = a;
       v[i] = a;
     }
@@ -134,10 +148,14 @@ int tl_depth_average(float* x, float* kept, const float* c, int t, long long tot
   return 0;
 }
 
-// x += LN(z + bias; w1, b1); with w2: out = LN(x; w2, b2).  Rows of a multiple of 4 up to 8,192 channels,
-// 16-byte aligned (the caller takes the norms one by one for any other).
+// x += LN(z + bias; w1, b1); with kept: kept[t] = x, x = sum_{j <= t} coef[j] kept[j] (kept float [> t, n, H]); with w2:
+// out = LN(x; w2, b2).  Rows of a multiple of 4 up to 8,192 channels, 16-byte aligned (the caller takes the steps one
+// by one for any other).
 int tl_layernorm_add_norm(const float* z, const float* bias, const float* w1, const float* b1, float eps1, float* x,
-                          const float* w2, const float* b2, float eps2, void* out, int out_dt, int n, int H, hipStream_t st) {
+                          const float* w2, const float* b2, float eps2, void* out, int out_dt, int n, int H, float* kept,
+                          const float* coef, int t, hipStream_t st) {
+  TL_REQUIRE(kept == nullptr || (coef != nullptr && t >= 0 && (uintptr_t)kept % 16 == 0), "layernorm_add_norm: versions of the stream without weights");
+  const long long total = (long long)n * H;
   TL_REQUIRE(n >= 0 && H > 0, "layernorm_add_norm: bad sizes n=%d H=%d", n, H);
   TL_REQUIRE(z && w1 && x && (w2 == nullptr || out != nullptr), "layernorm_add_norm: a buffer is missing");
   TL_REQUIRE(out_dt == DT_F32 || out_dt == DT_BF16, "layernorm_add_norm: unknown dtype code %d", out_dt);
@@ -148,8 +166,8 @@ int tl_layernorm_add_norm(const float* z, const float* bias, const float* w1, co
   const bool f32 = out_dt == DT_F32;
 #define TL_LAN(IT)                                                                                                          \
   do {                                                                                                                      \
-    if (f32) layernorm_add_norm_kernel<float, IT><<<n, 256, 0, st>>>(z, bias, w1, b1, eps1, x, w2, b2, eps2, (float*)out, H); \
-    else layernorm_add_norm_kernel<bf16, IT><<<n, 256, 0, st>>>(z, bias, w1, b1, eps1, x, w2, b2, eps2, (bf16*)out, H);       \
+    if (f32) layernorm_add_norm_kernel<float, IT><<<n, 256, 0, st>>>(z, bias, w1, b1, eps1, x, w2, b2, eps2, (float*)out, H, kept, coef, t, total); \
+    else layernorm_add_norm_kernel<bf16, IT><<<n, 256, 0, st>>>(z, bias, w1, b1, eps1, x, w2, b2, eps2, (bf16*)out, H, kept, coef, t, total);       \
   } while (0)
   if (H <= 1024) TL_LAN(1);
   else if (H <= 2048) TL_LAN(2);

@@ -144,25 +144,33 @@ class Model:
             self.embedding.forward(ctx, ctx.tokens, embedded)
         schedule = self.spec.schedule
         order = [self.blocks[run.layer] for run in schedule]
+        handed = False                       # the block before saw to this run's stream part
         for i, (block, binding) in enumerate(zip(order, runs)):
-            if schedule[i].entry is not None:
+            if schedule[i].entry is not None and not handed:
                 part, t = schedule[i].entry
                 flush_pending(ctx, x)
                 ctx.prenormed = None
                 self.stream_parts[part].forward(ctx, x, embedded, t)
+            # what changes the stream behind this block: a part whose change a norm's kernel can do is handed
+            # to a block that completes the stream with such a norm
+            nxt = schedule[i + 1].entry if i + 1 < len(order) else self.spec.exit
+            handed = (nxt is not None and getattr(block, "fuses_stream_after", False)
+                      and hasattr(self.stream_parts[nxt[0]], "mix_terms"))
             # the norm that reads the stream next, unless the stream changes before it does
             after = (order[i + 1].entry_norm()
-                     if i + 1 < len(order) and hasattr(order[i + 1], "entry_norm") and schedule[i + 1].entry is None
+                     if i + 1 < len(order) and hasattr(order[i + 1], "entry_norm") and (schedule[i + 1].entry is None or handed)
                      else None)
+            kw = {}
             if after is not None:
-                block.forward(ctx, binding, x, norm_after=after)
-            else:
-                block.forward(ctx, binding, x)
+                kw["norm_after"] = after
+            if handed:
+                kw["stream_after"] = (self.stream_parts[nxt[0]], nxt[1])
+            block.forward(ctx, binding, x, **kw)
         ctx.prenormed = None                 # nothing reads a norm's first half past the last block
         for commit in ctx.host.pop("deferred", []):
             commit()
         flush_pending(ctx, x)
-        if self.spec.exit is not None:
+        if self.spec.exit is not None and not handed:
             part, t = self.spec.exit
             self.stream_parts[part].forward(ctx, x, embedded, t)
         logits = ws.get("logits", (n_want, V), torch.float32)

@@ -376,10 +376,11 @@ def layernorm_rows_in_registers(H: int) -> bool:
 
 
 def layernorm_add_norm(z: torch.Tensor, w: torch.Tensor, beta, eps: float, x: torch.Tensor, bias=None,
-                       w_next=None, beta_next=None, eps_next: float = 0.0, out=None) -> None:
+                       w_next=None, beta_next=None, eps_next: float = 0.0, out=None, mix=None) -> None:
     """x += LN(z + bias; w, beta) and, with `w_next`, out = LN(x; w_next, beta_next) of the new row, in one
     kernel that holds the row in registers (`layernorm_rows_in_registers`).  z, x float32 [n, H]; out
-    [n, H] float32 or the compute dtype."""
+    [n, H] float32 or the compute dtype.  `mix` = (kept, coef, t): between the two, what `depth_average` does:
+    the new x is kept as version t and replaced by the weighted sum of versions 0 .. t."""
     n, H = z.shape
     _req(z, "layernorm_add_norm.z", torch.float32)
     _req(x, "layernorm_add_norm.x", torch.float32, (n, H))
@@ -388,10 +389,20 @@ def layernorm_add_norm(z: torch.Tensor, w: torch.Tensor, beta, eps: float, x: to
             _req(t, "layernorm_add_norm." + name, torch.float32, (H,))
     if w_next is not None:
         _req(out, "layernorm_add_norm.out", None, (n, H))
+    kept = coef = None
+    t = 0
+    if mix is not None:
+        kept, coef, t = mix
+        _req(kept, "layernorm_add_norm.kept", torch.float32)
+        _req(coef, "layernorm_add_norm.coef", torch.float32)
+        if kept.dim() != 3 or tuple(kept.shape[1:]) != (n, H) or kept.shape[0] <= t or coef.numel() <= t or t < 0:
+            raise KernelError(f"layernorm_add_norm: version {t} of a stream {(n, H)} in {tuple(kept.shape)} with "
+                              f"{coef.numel()} weights")
     _check(lib().tl_layernorm_add_norm(_p(z), _p(bias), _p(w), _p(beta), ctypes.c_float(eps), _p(x), _p(w_next),
                                        _p(beta_next) if w_next is not None else None, ctypes.c_float(eps_next),
                                        _p(out) if w_next is not None else None,
-                                       _code(out.dtype) if w_next is not None else DT_F32, n, H, _stream()))
+                                       _code(out.dtype) if w_next is not None else DT_F32, n, H, _p(kept), _p(coef), int(t),
+                                       _stream()))
 
 
 def depth_average(x: torch.Tensor, kept: torch.Tensor, coef: torch.Tensor, t: int) -> None:

@@ -189,7 +189,13 @@ class Norm(Part):
 
 
 class StreamPart(Part):
-    """A part that changes the residual stream between two runs of the schedule (`Run.entry`)."""
+    """A part that changes the residual stream between two runs of the schedule (`Run.entry`).
+
+    A part may also offer `mix_terms(ctx, x, t)`: the operands of its change, for the norm that
+    completes the stream before it (`Norm.add_to`'s `between`, a norm with `takes_between`) to do the
+    change in its own kernel.  A block that sets `fuses_stream_after` is then handed the part as
+    `stream_after=(part, t)` and sees to the change itself, in that norm's kernel or by calling
+    `part.forward`; the model does not call the part for that entry."""
     needs_embedding = False       # True: `forward` is handed the embedding's output of this step
 
     def forward(self, ctx: "StepContext", x: torch.Tensor, embedded: Optional[torch.Tensor], t: int) -> None:

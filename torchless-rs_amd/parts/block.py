@@ -217,7 +217,24 @@ class SandwichNormBlock(Part):
         may run it on the way (`Norm.add_to`'s `then`)."""
         return self.mixer_norm
 
-    def forward(self, ctx, run, x: torch.Tensor, norm_after=None) -> None:
+    fuses_stream_after = True     # takes `stream_after`: see `StreamPart`
+
+    def _last_add(self, ctx, norm, z, x, bias, y, norm_after, stream_after) -> None:
+        """The block's last norm into the stream, with what changes the stream behind the block."""
+        then = None if norm_after is None else (norm_after, y)
+        if stream_after is None:
+            norm.add_to(ctx, z, x, bias=bias, then=then)
+            return
+        part, t = stream_after
+        if getattr(norm, "takes_between", False):
+            norm.add_to(ctx, z, x, bias=bias, then=then, between=part.mix_terms(ctx, x, t))
+        else:
+            norm.add_to(ctx, z, x, bias=bias)
+            part.forward(ctx, x, None, t)
+
+    def forward(self, ctx, run, x: torch.Tensor, norm_after=None, stream_after=None) -> None:
+        """`stream_after` = (stream part, t): that part changes the stream right behind this block; the
+        block's last norm does it on its way if it can, and `norm_after` then reads the changed stream."""
         ctx.host.pop("stream_copy", None)        # this block writes the stream: a copy of it goes stale
         ws = ctx.workspace
         y = ws.get("block_y", tuple(x.shape), ctx.dtype)
@@ -225,14 +242,14 @@ class SandwichNormBlock(Part):
         y1 = read_through_norm(ctx, self.mixer_norm, x, y)
         take_row_factor(ctx, usable=False)       # a norm cut in two by an earlier product is completed here
         bias = OutputNormBlock._result(ctx, self.mixer, z, run, y1)
-        after = self.ffn_norm if self.ffn is not None else norm_after
-        self.mixer_out_norm.add_to(ctx, z, x, bias=bias, then=None if after is None else (after, y))
         if self.ffn is None:
+            self._last_add(ctx, self.mixer_out_norm, z, x, bias, y, norm_after, stream_after)
             return
+        self.mixer_out_norm.add_to(ctx, z, x, bias=bias, then=(self.ffn_norm, y))
         y2 = read_through_norm(ctx, self.ffn_norm, x, y)
         take_row_factor(ctx, usable=False)
         bias = OutputNormBlock._result(ctx, self.ffn, z, y2)
-        self.ffn_out_norm.add_to(ctx, z, x, bias=bias, then=None if norm_after is None else (norm_after, y))
+        self._last_add(ctx, self.ffn_out_norm, z, x, bias, y, norm_after, stream_after)
 
 
 register_part("block", "pre_norm", PreNormBlock)

@@ -99,17 +99,28 @@ class LayerNorm(Norm):
             ctx.pending = None
         ops.layernorm(x, self.weight, self.eps, out, beta=self.beta)
 
-    def add_to(self, ctx, z: torch.Tensor, x: torch.Tensor, out=None, bias=None, then=None) -> None:
+    takes_between = True          # `add_to` may be handed what a stream part does between this norm and the next
+
+    def add_to(self, ctx, z: torch.Tensor, x: torch.Tensor, out=None, bias=None, then=None, between=None) -> None:
+        """`between` = (kept, coef, t) (`ops.depth_average`'s operands): the stream's new version is kept and
+        replaced by the weighted sum of its versions before `then`'s norm reads it."""
         nxt = then[0] if then is not None and isinstance(then[0], LayerNorm) and then[0].size == self.size else None
         if out is None and ops.layernorm_rows_in_registers(self.size):
             if nxt is not None:
                 ops.layernorm_add_norm(z, self.weight, self.beta, self.eps, x, bias=bias, w_next=nxt.weight,
-                                       beta_next=nxt.beta, eps_next=nxt.eps, out=then[1])
+                                       beta_next=nxt.beta, eps_next=nxt.eps, out=then[1], mix=between)
                 ctx.prenormed = (nxt, then[1], None)
             else:
-                ops.layernorm_add_norm(z, self.weight, self.beta, self.eps, x, bias=bias)
+                ops.layernorm_add_norm(z, self.weight, self.beta, self.eps, x, bias=bias, mix=between)
             return
         ops.layernorm(z, self.weight, self.eps, out, add_to=x, bias=bias, beta=self.beta)
+        if between is not None:
+            ops.depth_average(x, *between)
+            if out is not None:
+                if out.dtype == torch.float32:
+                    out.copy_(x)
+                else:
+                    ops.cast_rows(x, out)
 
 
 register_part("norm", "rmsnorm", RMSNorm)

@@ -39,11 +39,16 @@ class DepthAverage(StreamPart):
         self.coef = [tensors[name].to(torch.float32).contiguous() for name in self.names]
         self.one = torch.ones(1, dtype=torch.float32, device=self.coef[0].device) if self.coef else None
 
-    def forward(self, ctx, x: torch.Tensor, embedded, t: int) -> None:
+    def mix_terms(self, ctx, x: torch.Tensor, t: int):
+        """(kept, weights, t): the operands of `ops.depth_average` for call t, for a norm whose kernel
+        does the sum on its way (`Norm.add_to`'s `between`)."""
         if not (0 <= t <= len(self.names)):
             raise ValueError(f"average {t} of {len(self.names)}")
         kept = ctx.workspace.get("depth_kept", (len(self.names) + 1,) + tuple(x.shape), torch.float32)
-        ops.depth_average(x, kept, self.one if t == 0 else self.coef[t - 1], t)
+        return kept, (self.one if t == 0 else self.coef[t - 1]), t
+
+    def forward(self, ctx, x: torch.Tensor, embedded, t: int) -> None:
+        ops.depth_average(x, *self.mix_terms(ctx, x, t))
 
 
 register_part("stream", "depth_average", DepthAverage)
