@@ -6,7 +6,7 @@ Notation.  x: the residual stream [T, W].  ln(t, w, b) = (t - mean) / sqrt(var +
 the last axis.  A layer is x <- x + ln1b(mixer(ln1(x))); x <- x + ln2b(ff(ln2(x))) (the second only
 with a feed-forward); then the stream that goes on is a weighted sum of the embedding's output
 and every layer's result so far.  Mixers: grouped-query attention whose weights are logistic
-functions of the scores (no softmax) inside chunks of positions, and a gated recurrence per
+functions of the scores, each key by itself, inside chunks of positions, and a gated recurrence per
 channel.  Feed-forward: a routed mixture of small gated experts, the router's weight on an
 expert's input, with a shared expert.
 """

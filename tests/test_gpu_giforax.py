@@ -259,7 +259,7 @@ def test_a_state_that_is_carried_far_and_one_that_is_forgotten(by_runs):
 # ---------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("in_dtype", DTYPES)
-@pytest.mark.parametrize("E, top", [(8, 2), (12, 1), (1, 1), (4, 4), (40, 7)])
+@pytest.mark.parametrize("E, top", [(8, 2), (10, 1), (1, 1), (4, 4), (40, 7)])
 def test_the_router_with_a_score_of_its_own_for_every_expert(in_dtype, E, top):
     from torchless_rs_amd.kernels import ops
     g = torch.Generator().manual_seed(E * 10 + top)
@@ -293,7 +293,7 @@ def experts_part(dtype, H, E, top, ff, limit, shared, on, seed):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H, E, top, ff, limit, shared", [(64, 8, 2, 32, 1.5, (48, 0.75)), (100, 5, 2, 12, 1.0, (10, 2.0)),
-                                                          (32, 1, 1, 16, 0.5, None), (48, 12, 1, 8, 2.0, (8, 2.0)), (40, 4, 4, 8, 1.0, None)])
+                                                          (32, 1, 1, 16, 0.5, None), (48, 10, 1, 8, 2.0, (8, 2.0)), (40, 4, 4, 8, 1.0, None)])
 def test_gated_experts_with_the_weight_on_their_input(dtype, H, E, top, ff, limit, shared):
     """The chosen experts alone (few rows), all experts side by side (more rows) and, in bfloat16, expert by expert over
     each expert's own rows, against the plain mixture; clamps that bite (weights with a gain of 3), a shared expert with

@@ -1,4 +1,4 @@
-// A gated recurrence per channel whose gates read the current row alone:
+// A recurrence per channel whose update gate z and candidate c are functions of the present row only:
 //
 //     z_t = logistic(a_t + bz) ,  c_t = cand(b_t + bx) ,  S_t = (1 - z_t) S_(t-1) + z_t c_t ,
 //     out_t = S_t * silu(g_t)

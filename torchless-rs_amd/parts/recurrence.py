@@ -1,4 +1,5 @@
-"""A gated recurrence per channel whose gates read the current token alone (a minimal GRU).
+"""A recurrence per channel with an update gate and a candidate that are functions of the present row
+only (the smallest of the gated recurrent units): nothing of the state enters its gates.
 
 With `width` channels, one product over the mixer's input y gives a row [a | b | g], and per
 channel
