@@ -18,18 +18,20 @@ namespace tl {
 
 constexpr int RT_MAX_E = 1024;
 
-template <typename T>
-__global__ void __launch_bounds__(256)
+// NT threads a row: a quarter of a thousand, or 1024 for steps of few rows, where a row's dots are what the step waits
+// for (16 waves take 16 experts at a time instead of 4).  A dot is one wave's either way: the same bits.
+template <typename T, int NT>
+__global__ void __launch_bounds__(NT)
 route_kernel(const T* __restrict__ h, int W, const float* __restrict__ wr, int E, int groups, int keep, int top,
              int logistic, float* __restrict__ weights, int* __restrict__ chosen, bool vec) {
   __shared__ float s_s[RT_MAX_E];
   __shared__ float g_s[RT_MAX_E];
   __shared__ unsigned char ok_s[RT_MAX_E];
-  __shared__ float sh[4];
+  __shared__ float sh[NT / WAVE];
   const int n = blockIdx.x;
   const int t = threadIdx.x, lane = t % WAVE, wave = t / WAVE;
   const T* row = h + (size_t)n * W;
-  for (int e = wave; e < E; e += 4) {
+  for (int e = wave; e < E; e += NT / WAVE) {
     const float* w = wr + (size_t)e * W;
     float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;      // four chains: the loads of one do not wait for another's sum
     int c = 0;
@@ -58,37 +60,37 @@ route_kernel(const T* __restrict__ h, int W, const float* __restrict__ wr, int E
   }
   __syncthreads();
   if (logistic) {                                      // every expert's score by itself
-    for (int e = t; e < E; e += 256) s_s[e] = 1.0f / (1.0f + expf(-s_s[e]));
+    for (int e = t; e < E; e += NT) s_s[e] = 1.0f / (1.0f + expf(-s_s[e]));
   } else {
     float m = -INFINITY;
-    for (int e = t; e < E; e += 256) m = fmaxf(m, s_s[e]);
-    m = block_max<256>(m, sh);
+    for (int e = t; e < E; e += NT) m = fmaxf(m, s_s[e]);
+    m = block_max<NT>(m, sh);
     float sum = 0.f;
-    for (int e = t; e < E; e += 256) sum += expf(s_s[e] - m);
-    sum = block_sum<256>(sum, sh);
+    for (int e = t; e < E; e += NT) sum += expf(s_s[e] - m);
+    sum = block_sum<NT>(sum, sh);
     __syncthreads();
-    for (int e = t; e < E; e += 256) s_s[e] = expf(s_s[e] - m) / sum;
+    for (int e = t; e < E; e += NT) s_s[e] = expf(s_s[e] - m) / sum;
   }
   __syncthreads();
   if (groups > 0) {
     const int per = E / groups;
-    for (int g = t; g < groups; g += 256) {
+    for (int g = t; g < groups; g += NT) {
       float best = s_s[g * per];
       for (int i = 1; i < per; ++i) best = fmaxf(best, s_s[g * per + i]);
       g_s[g] = best;
     }
     __syncthreads();
-    for (int g = t; g < groups; g += 256) {
+    for (int g = t; g < groups; g += NT) {
       int ahead = 0;
       const float mine = g_s[g];
       for (int o = 0; o < groups; ++o) ahead += (g_s[o] > mine || (g_s[o] == mine && o < g)) ? 1 : 0;
       for (int i = 0; i < per; ++i) ok_s[g * per + i] = ahead < keep;
     }
   } else {
-    for (int e = t; e < E; e += 256) ok_s[e] = 1;
+    for (int e = t; e < E; e += NT) ok_s[e] = 1;
   }
   __syncthreads();
-  for (int e = t; e < E; e += 256) {
+  for (int e = t; e < E; e += NT) {
     float wgt = 0.f;
     if (ok_s[e]) {
       int ahead = 0;
@@ -307,12 +309,16 @@ int tl_route(const void* h, int dt, int n, int W, const float* wr, int E, int gr
   TL_REQUIRE(h && wr && weights, "route: a buffer is missing");
   if (n == 0) return 0;
   const bool vec = W % 4 == 0 && (uintptr_t)h % 16 == 0 && (uintptr_t)wr % 16 == 0;
-  if (dt == DT_F32)
-    route_kernel<float><<<n, 256, 0, st>>>((const float*)h, W, wr, E, groups, keep, top, logistic, weights, chosen, vec);
-  else if (dt == DT_BF16)
-    route_kernel<bf16><<<n, 256, 0, st>>>((const bf16*)h, W, wr, E, groups, keep, top, logistic, weights, chosen, vec);
+  TL_REQUIRE(dt == DT_F32 || dt == DT_BF16, "route: unknown dtype code %d", dt);
+  const bool few = n <= 64 && E > 4;             // fewer rows than compute units: more waves a row
+  if (dt == DT_F32 && few)
+    route_kernel<float, 1024><<<n, 1024, 0, st>>>((const float*)h, W, wr, E, groups, keep, top, logistic, weights, chosen, vec);
+  else if (dt == DT_F32)
+    route_kernel<float, 256><<<n, 256, 0, st>>>((const float*)h, W, wr, E, groups, keep, top, logistic, weights, chosen, vec);
+  else if (few)
+    route_kernel<bf16, 1024><<<n, 1024, 0, st>>>((const bf16*)h, W, wr, E, groups, keep, top, logistic, weights, chosen, vec);
   else
-    TL_REQUIRE(false, "route: unknown dtype code %d", dt);
+    route_kernel<bf16, 256><<<n, 256, 0, st>>>((const bf16*)h, W, wr, E, groups, keep, top, logistic, weights, chosen, vec);
   TL_LAUNCH_CHECK("route");
   return 0;
 }
