@@ -809,3 +809,79 @@ def test_the_command_line_and_the_trace_replay(zoo, tmp_path):
     want = z["want"][2]
     assert rel_err(first, torch.stack([want[0], want[19], want[2]])) < TOL["float32"]
     assert rel_err(last, want[21:22]) < TOL["float32"]
+
+
+# ---------------------------------------------------------------------------------------------
+# configurations drawn at random
+# ---------------------------------------------------------------------------------------------
+
+def random_config(rng):
+    """Any order of layers, any sizes: recurrences of 8 to 384 channels, heads of 16 to 128 with values as wide or not,
+    one to four KV heads, none, half or all of a head rotated, no chunks or chunks of 17 to 256, readers of any earlier
+    layer that owns keys (with more heads and another chunk), one to sixteen experts with or without a shared one."""
+    width = rng.choice([64, 96, 128, 160, 256])
+    layers, owners = [], []
+    for i in range(rng.randint(3, 6)):
+        if rng.random() < 0.3:
+            mix = gru(rng.choice([8, 33, 64, 200, 384]))
+        elif owners and rng.random() < 0.35:
+            src = rng.choice(owners)
+            m0 = layers[src]["mixer"]
+            mix = attn(m0["kv_heads"] * rng.choice([1, 2, 4]), m0["kv_heads"], m0["dim"], m0["vdim"], rng.uniform(0.08, 0.3),
+                       rot=(m0["rot"]["base"], m0["rot"]["dims"]) if "rot" in m0 else None,
+                       chunk=rng.choice([None, 17, 64, 100, 200, 256]), kv_from=src)
+        else:
+            dim = rng.choice([16, 32, 48, 64, 96, 128])
+            kv = rng.choice([1, 2, 4])
+            dims = rng.choice([0, dim // 2, dim])
+            mix = attn(kv * rng.choice([1, 2, 4]), kv, dim, dim if rng.random() < 0.7 else rng.choice([16, 24, 64]),
+                       rng.uniform(0.08, 0.3), rot=(rng.choice([100.0, 10000.0, 5e5]), dims) if dims else None,
+                       chunk=rng.choice([None, 17, 64, 100, 200, 256]))
+            owners.append(i)
+        f = None
+        if rng.random() < 0.85:
+            E = rng.choice([1, 2, 4, 8, 10, 16])
+            f = moe(E, rng.randint(1, min(E, 4)), rng.choice([8, 16, 32, 64]), rng.choice([0.5, 1.5, 3.0]),
+                    shared=(rng.choice([8, 32, 96]), rng.choice([0.5, 1.5])) if rng.random() < 0.7 else None)
+        layers.append(layer(mix, f))
+    return model(rng.choice([97, 256, 500]), width, rng.choice([1e-5, 1e-6]), rng.choice([0.5, 1.0, 2.0]), layers)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_configurations(seed, tmp_path):
+    """Float32 (where a router's choice falls the same way as in the plain implementation): whole prompts, a prompt
+    with its last tokens one by one, and all of them in one batch that is decoded together."""
+    import random
+    from torchless_rs_amd.engine import Engine, SeqInput, load_model
+    cfg = random_config(random.Random(seed))
+    w = plain.random_weights(cfg, seed=100 + seed)
+    ps = some_prompts(cfg["vocab"], [1, 37, 150, 420], seed=seed)
+    runs = [plain_run(w, cfg, p) for p in ps]
+    eng = Engine(load_model(write_model(str(tmp_path / "m"), cfg, w), "float32"), max_tokens=64 * 30, max_slots=8)
+    tails = [0, 5, 20, 33]
+    heads = [len(p) - t for p, t in zip(ps, tails)]
+    for p, h, (want, m) in zip(ps, heads, runs):
+        s = eng.alloc()
+        got = eng.step([SeqInput(s, p, list(range(len(p))))]).clone()
+        eng.free(s)
+        close(got, want, "float32", (seed, len(p), "whole"), m)
+        s = eng.alloc()
+        rows = [eng.step([SeqInput(s, p[:h], list(range(h)))]).clone()] + [eng.step([SeqInput(s, [t], [0])]).clone() for t in p[h:]]
+        eng.free(s)
+        close(torch.cat(rows), want, "float32", (seed, len(p), "then decoded"), m)
+    slots = [eng.alloc() for _ in ps]
+    lg = eng.step([SeqInput(s, p[:h], list(range(h))) for s, p, h in zip(slots, ps, heads)])
+    got, at = [], 0
+    for h in heads:
+        got.append([lg[at:at + h].clone()])
+        at += h
+    for step in range(max(tails)):
+        live = [i for i in range(len(ps)) if step < tails[i]]
+        lg = eng.step([SeqInput(slots[i], [ps[i][heads[i] + step]], [0]) for i in live]).clone()
+        for r, i in enumerate(live):
+            got[i].append(lg[r:r + 1])
+    for s in slots:
+        eng.free(s)
+    for i, (want, m) in enumerate(runs):
+        close(torch.cat(got[i]), want, "float32", (seed, i, "together"), m)
+    eng.close()
